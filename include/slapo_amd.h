@@ -1,0 +1,181 @@
+/*
+ * slapo_amd.h -- C ABI of libslapo_amd.so: the gfx950 (MI355X / CDNA4) kernels behind
+ * Slapo's fused-op hot path (slapo.op attention + FusedMLP epilogues + dropout RNG).
+ *
+ * The reference (awslabs/slapo) is pure Python and has no FFI of its own: the points where it
+ * leaves Python for a fused kernel are third-party calls.  Every entry point below names the
+ * reference call site whose callee it replaces.  All entry points
+ *   - take plain device pointers, sizes, strides and a hipStream_t passed as void*;
+ *   - never allocate or free memory (workspaces are caller-provided);
+ *   - are stateless and re-entrant; they enqueue work on `stream` and return without
+ *     synchronising;
+ *   - return 0 on success or a negative SLAPO_ERR_* code (see slapo_amd_status_string).
+ *
+ * Tensors: q/k/v/o/do/dq/dk/dv are logically [batch, seqlen, heads, head_dim] with head_dim
+ * contiguous; the three outer strides are given in elements, so the fused-QKV GEMM output
+ * ([B,S,H,3D] view, reference slapo/op/attention.py:469-481) can be consumed without copies.
+ */
+#ifndef SLAPO_AMD_H
+#define SLAPO_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SLAPO_AMD_ABI_VERSION 1
+
+/* status codes */
+#define SLAPO_OK 0
+#define SLAPO_ERR_DTYPE (-1)     /* unsupported element type                               */
+#define SLAPO_ERR_SHAPE (-2)     /* unsupported / inconsistent sizes (e.g. head_dim > 128) */
+#define SLAPO_ERR_ALIGN (-3)     /* pointer or stride not aligned as the kernel requires   */
+#define SLAPO_ERR_ARG (-4)       /* null pointer / out-of-range scalar argument            */
+#define SLAPO_ERR_LAUNCH (-5)    /* hipLaunch / hipGetLastError reported a failure         */
+#define SLAPO_ERR_DEVICE (-6)    /* no usable gfx950 device                                */
+#define SLAPO_ERR_WORKSPACE (-7) /* caller workspace missing or too small                  */
+
+/* element types */
+#define SLAPO_F32 0
+#define SLAPO_F16 1
+#define SLAPO_BF16 2
+
+int slapo_amd_abi_version(void);
+const char* slapo_amd_status_string(int status);
+
+/* ------------------------------------------------------------------------------------------
+ * Dropout RNG (Philox4x32-10 with ATen's element <-> (subsequence, counter, lane) mapping).
+ *
+ * Replaces: the ATen native_dropout launch reached from torch.nn.functional.dropout at
+ * slapo/op/fused_bias.py:74 (bias_dropout) and slapo/op/attention.py:179-180 (xformers_ref).
+ * The mask is a pure function of (seed, offset, plan), so it can be regenerated in backward
+ * and under activation-checkpoint recompute (slapo/checkpoint.py:79-92).
+ * ---------------------------------------------------------------------------------------- */
+typedef struct slapo_dropout_plan {
+    int64_t numel;            /* elements of the tensor the mask is drawn for                  */
+    int64_t total_threads;    /* T = 256 * grid: Philox subsequences in use                     */
+    int32_t vec;              /* elements handled per subsequence per loop trip: 1,2,4,8,16     */
+    int32_t calls_per_iter;   /* Philox calls per loop trip = ceil(vec/4) (1 when vec == 1)     */
+    int64_t offset_increment; /* amount the generator's offset must be advanced after the draw */
+} slapo_dropout_plan;
+
+/* Host Philox4x32-10 block function (10 rounds).  Pure host code; usable without a GPU. */
+void slapo_amd_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4]);
+
+/* Launch geometry ATen would choose for a dense tensor of `numel` elements of `elem_bytes`
+ * bytes whose data pointer is aligned to `ptr_align` bytes, on a device with `num_cus`
+ * compute units and `max_threads_per_cu` resident threads per CU.  Pure host code. */
+int slapo_amd_dropout_plan_for(int64_t numel, int elem_bytes, int64_t ptr_align, int num_cus,
+                               int max_threads_per_cu, slapo_dropout_plan* plan);
+
+/* Same, reading num_cus / max_threads_per_cu from HIP device `device`. */
+int slapo_amd_dropout_plan(int64_t numel, int elem_bytes, int64_t ptr_align, int device,
+                           slapo_dropout_plan* plan);
+
+/* Largest 32-bit Philox output that is KEPT for drop probability p (keep iff
+ * 2^-32 + float(v) * 2^-32 < (float)(1.0 - p)); *keep_all is set when every output is kept and
+ * *keep_none when none is.  Pure host code. */
+uint32_t slapo_amd_dropout_threshold(double p, int* keep_all, int* keep_none);
+
+/* Host mirror: mask[i] = 1 if element i is kept.  Pure host code (test / debugging aid). */
+int slapo_amd_dropout_mask_host(uint8_t* mask, const slapo_dropout_plan* plan, double p,
+                                uint64_t seed, uint64_t offset);
+
+/* Device version of the same (mask is a device pointer to numel bytes). */
+int slapo_amd_dropout_mask(uint8_t* mask, const slapo_dropout_plan* plan, double p,
+                           uint64_t seed, uint64_t offset, void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * FusedMLP epilogues.  x / y / out / grads are [rows, cols] row-major with row stride == cols;
+ * bias is [cols].  dtype is one of SLAPO_F32 / SLAPO_F16 / SLAPO_BF16 for all tensors of a call.
+ * ---------------------------------------------------------------------------------------- */
+
+/* out = gelu_tanh(y + bias).
+ * Replaces: BiasGeLUFunction.bias_gelu (slapo/op/fused_bias.py:18-21) reached from
+ * LinearWithAct.forward (slapo/op/linear.py:184-188); also bias_new_gelu (fused_bias.py:63-64). */
+int slapo_amd_bias_gelu_fwd(const void* y, const void* bias, void* out, int64_t rows,
+                            int64_t cols, int dtype, void* stream);
+
+/* Bytes of fp32 workspace the two backward epilogues need for the column (bias) reduction. */
+size_t slapo_amd_colsum_workspace_bytes(int64_t rows, int64_t cols);
+
+/* dx = dgelu_tanh(y + bias) * grad;  dbias[c] = sum_r dx[r, c]  (dbias may be NULL).
+ * Replaces: BiasGeLUFunction.bias_gelu_back + autograd's broadcast reduction of the bias
+ * gradient (slapo/op/fused_bias.py:26-34, 42-46). */
+int slapo_amd_bias_gelu_bwd(const void* grad, const void* y, const void* bias, void* dx,
+                            void* dbias, void* workspace, size_t workspace_bytes, int64_t rows,
+                            int64_t cols, int dtype, void* stream);
+
+/* out = dropout(x + bias, p) [+ residual]   (residual may be NULL; p == 0 disables dropout).
+ * The mask is the one torch.nn.functional.dropout would draw for the [rows, cols] tensor under
+ * generator state (seed, offset) and launch plan `plan` (ignored when p == 0).
+ * Replaces: bias_dropout (slapo/op/fused_bias.py:67-74) reached from LinearWithDropout.forward
+ * (slapo/op/linear.py:252-258); with residual, the fusion pattern of tests/test_fusion.py:179-180. */
+int slapo_amd_bias_dropout_residual_fwd(const void* x, const void* bias, const void* residual,
+                                        void* out, int64_t rows, int64_t cols, int dtype,
+                                        double p, uint64_t seed, uint64_t offset,
+                                        const slapo_dropout_plan* plan, void* stream);
+
+/* dx = grad * mask / (1 - p);  dbias[c] = sum_r dx[r, c] (dbias may be NULL).  The residual
+ * gradient is `grad` itself and needs no kernel.  Replaces: autograd of the same pattern. */
+int slapo_amd_bias_dropout_residual_bwd(const void* grad, void* dx, void* dbias,
+                                        void* workspace, size_t workspace_bytes, int64_t rows,
+                                        int64_t cols, int dtype, double p, uint64_t seed,
+                                        uint64_t offset, const slapo_dropout_plan* plan,
+                                        void* stream);
+
+/* ------------------------------------------------------------------------------------------
+ * Attention:  O = dropout(softmax(Q K^T * scale + bias + mask)) V, forward and backward.
+ *
+ * Replaces: the attn_fn callees of FlashAttentionOp.forward -- xformers
+ * memory_efficient_attention (slapo/op/attention.py:315), flash-attn Triton flash_attn_func
+ * (:328-336) and flash_attn_unpadded_func (:353-364); semantics pinned by the native
+ * restatements xformers_ref (:134-196) and flash_attn_ref (:39-131).
+ * ---------------------------------------------------------------------------------------- */
+typedef struct slapo_attn_params {
+    int32_t dtype;    /* SLAPO_F16 / SLAPO_BF16 (MFMA kernels) or SLAPO_F32 (fp32 FMA kernels)  */
+    int32_t batch;
+    int32_t heads;
+    int32_t seqlen_q;
+    int32_t seqlen_k;
+    int32_t head_dim; /* <= 128 and a multiple of 8 for 16-bit types; <= 128 for fp32           */
+    int32_t causal;   /* key j visible to query i only if j <= i                                */
+    int32_t window;   /* > 0: additionally i - j < window (local causal attention); 0 = off     */
+    float scale;      /* softmax scale (reference default head_dim^-0.5)                        */
+    float p_drop;     /* dropout probability on the attention matrix; 0 disables                */
+    uint64_t seed;    /* Philox seed (generator seed)                                           */
+    uint64_t offset;  /* Philox offset (generator offset at entry of forward)                   */
+    /* element strides of [batch, seqlen, heads] for each tensor; head_dim stride is 1 */
+    int64_t q_strides[3];
+    int64_t k_strides[3];
+    int64_t v_strides[3];
+    int64_t o_strides[3];
+    /* additive fp32 bias addressed as bias[b*s0 + h*s1 + i*s2 + j*s3]; stride 0 broadcasts
+     * (the reference's "b11k" layout is {Sk, 0, 0, 1}, "bhqk" is {H*Sq*Sk, Sq*Sk, Sk, 1}) */
+    int64_t bias_strides[4];
+    /* launch plan of the dropout mask over the dense [batch*heads, seqlen_q, seqlen_k] fp32
+     * probability tensor (only read when p_drop > 0) */
+    slapo_dropout_plan plan;
+} slapo_attn_params;
+
+/* lse: [batch, heads, seqlen_q] fp32, natural-log sum-exp of the masked, scaled scores. */
+int slapo_amd_attn_fwd(const slapo_attn_params* prm, const void* q, const void* k, const void* v,
+                       const float* bias, void* o, float* lse, void* stream);
+
+/* Workspace (bytes) the backward needs: fp32 dQ accumulator + fp32 delta = rowsum(dO * O). */
+size_t slapo_amd_attn_bwd_workspace_bytes(const slapo_attn_params* prm);
+
+/* dq/dk/dv use q_strides/k_strides/v_strides of a DENSE [B,S,H,D] layout given in
+ * dq_strides/dk_strides/dv_strides; `dout` uses o_strides. */
+int slapo_amd_attn_bwd(const slapo_attn_params* prm, const void* q, const void* k, const void* v,
+                       const float* bias, const void* o, const void* dout, const float* lse,
+                       void* dq, void* dk, void* dv, const int64_t dq_strides[3],
+                       const int64_t dk_strides[3], const int64_t dv_strides[3], void* workspace,
+                       size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SLAPO_AMD_H */

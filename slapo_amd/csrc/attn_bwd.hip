@@ -1,0 +1,393 @@
+// Flash-attention backward for gfx950, fp16 / bf16 inputs, fp32 accumulation.
+//
+// One workgroup (4 wavefronts) owns 128 consecutive keys of one (batch, head); wavefront w owns
+// 32 of them and keeps their K and V fragments in registers for the whole kernel, together with
+// its dK^T and dV^T accumulators.  Query tiles of 32 rows (Q, dO, lse, delta) stream through LDS,
+// double buffered and staged through registers.  Per query tile and wavefront (lane l,
+// g = l / 32):
+//   S  = Q K_w^T, dP = dO V_w^T      A = Q / dO rows from LDS (row-permuted 128-bit reads),
+//                                    B = the resident K_w / V_w fragments.  Lane l holds one KEY
+//                                    column; registers run over 16 query rows.
+//   P  = exp2(S * scale - lse), dS = P * (dP - delta)      recomputed from the saved
+//                                    log-sum-exp; dropout bits regenerated from Philox.
+//   dV_w^T += dO^T P, dK_w^T += Q^T dS    B = P / dS straight from the accumulator registers
+//                                    (the row permutation makes them ordered k-slots), A = dO^T /
+//                                    Q^T read from the same row-major LDS tiles with the
+//                                    transposing LDS read.
+//   dQ += dS K                       dS goes through LDS once ([key][query], double buffered);
+//                                    after the barrier each wavefront computes 16 head-dim
+//                                    columns of dQ over ALL 128 keys of the workgroup with
+//                                    16x16x32 MFMAs (A = dS via the transposing read, B = K^T
+//                                    fragments resident in registers) and adds the tile into the
+//                                    fp32 dQ accumulator with hardware float atomics: one atomic
+//                                    tile per workgroup and query tile instead of one per
+//                                    wavefront.
+// One barrier per query tile.  Reference semantics: autograd of slapo/op/attention.py:163-181.
+#include <hip/amd_detail/amd_hip_unsafe_atomics.h>
+
+#include "attn_common.h"
+
+using namespace slapo;
+
+namespace {
+
+constexpr int kBwdWaves = 4;
+constexpr int kBwdThreads = kBwdWaves * 64;
+constexpr int kBwdBN = kBwdWaves * 32;  // keys per workgroup
+constexpr int kBwdBM = 32;              // queries per tile
+constexpr int kDsPitch = kBwdBM + 8;    // dS tile [key][query] row pitch (elements)
+
+template <typename T, int DPAD>
+struct BwdSmem {
+    typedef TileStage<T, DPAD, kBwdBM, kBwdThreads> QStage;
+    static constexpr int kPitch = QStage::kPitch;
+    static constexpr int kQTile = kBwdBM * kPitch;            // elements
+    static constexpr int kDsTile = kBwdBN * kDsPitch;         // elements
+    static constexpr int kKStage = kBwdBN * kPitch;           // elements (start-up only)
+    static constexpr size_t kQBytes = 2 * kQTile * sizeof(T);   // double buffered
+    static constexpr size_t kDsBytes = 2 * kDsTile * sizeof(T);
+    static constexpr size_t kStatBytes = 2 * 2 * kBwdBM * sizeof(float);
+    static constexpr size_t kLoopBytes = 2 * kQBytes + kDsBytes + kStatBytes;
+    static constexpr size_t kStageBytes = kKStage * sizeof(T);
+    static constexpr size_t kBytes = kLoopBytes > kStageBytes ? kLoopBytes : kStageBytes;
+};
+
+template <typename T, int DPAD>
+__global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_kernel(
+    const AttnArgs a) {
+    typedef typename Mma<T>::frag frag_t;
+    typedef BwdSmem<T, DPAD> SM;
+    typedef typename SM::QStage QStage;
+    constexpr int kPitch = SM::kPitch;
+    constexpr int DK = DPAD / 16;          // k-steps over head dim
+    constexpr int DV = DPAD / 32;          // 32-row blocks of dK^T / dV^T
+    constexpr int NBLK = DPAD / 16;        // 16-column blocks of dQ
+    constexpr int NDB = (NBLK + kBwdWaves - 1) / kBwdWaves;  // dQ blocks per wavefront
+
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    T* q_lds = reinterpret_cast<T*>(smem_raw);
+    T* g_lds = reinterpret_cast<T*>(smem_raw + SM::kQBytes);
+    T* ds_lds = reinterpret_cast<T*>(smem_raw + 2 * SM::kQBytes);
+    float* stat_lds = reinterpret_cast<float*>(smem_raw + 2 * SM::kQBytes + SM::kDsBytes);
+    T* kstage = reinterpret_cast<T*>(smem_raw);
+
+    const int n_bh = a.batch * a.heads;
+    const int bh = blockIdx.x % n_bh;
+    const int kt = blockIdx.x / n_bh;  // low key tiles see the most queries under a causal mask
+    const int b = bh / a.heads;
+    const int h = bh % a.heads;
+    const int k0 = kt * kBwdBN;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int g = lane >> 5;
+    const int c_loc = lane & 31;
+    const int kw0 = k0 + wave * 32;
+    const int key = kw0 + c_loc;  // this lane's key column
+
+    const T* q_base = reinterpret_cast<const T*>(a.q) + b * a.qs[0] + h * a.qs[2];
+    const T* k_base = reinterpret_cast<const T*>(a.k) + b * a.ks[0] + h * a.ks[2];
+    const T* v_base = reinterpret_cast<const T*>(a.v) + b * a.vs[0] + h * a.vs[2];
+    const T* g_base = reinterpret_cast<const T*>(a.dout) + b * a.os[0] + h * a.os[2];
+    const float* lse_base = a.lse + (int64_t)bh * a.sq;
+    const float* delta_base = a.delta + (int64_t)bh * a.sq;
+    float* dq_base = reinterpret_cast<float*>(a.dq) + (int64_t)bh * a.sq * a.d;
+
+    // ---- resident fragments ----
+    frag_t kf[DK], vf[DK];
+#pragma unroll
+    for (int t = 0; t < DK; ++t) {
+        u32x4_t kv = {0u, 0u, 0u, 0u}, vv = {0u, 0u, 0u, 0u};
+        const int d0 = 16 * t + 8 * g;
+        if (key < a.sk && d0 < a.d) {
+            kv = *reinterpret_cast<const u32x4_t*>(k_base + (int64_t)key * a.ks[1] + d0);
+            vv = *reinterpret_cast<const u32x4_t*>(v_base + (int64_t)key * a.vs[1] + d0);
+        }
+        kf[t] = __builtin_bit_cast(frag_t, kv);
+        vf[t] = __builtin_bit_cast(frag_t, vv);
+    }
+    // K^T fragments for dQ = dS K: B operand of the 16x16x32 MFMA, column d, k-slots = keys.
+    frag_t ktf[NDB][kBwdWaves];
+    {
+        TileStage<T, DPAD, kBwdBN, kBwdThreads> kst;
+        kst.load(k_base, a.ks[1], k0, a.sk, a.d);
+        kst.store(kstage);
+        __syncthreads();
+        const int beta = lane >> 4;
+#pragma unroll
+        for (int nb = 0; nb < NDB; ++nb) {
+            const int blk = wave + nb * kBwdWaves;
+#pragma unroll
+            for (int st = 0; st < kBwdWaves; ++st) {
+                if (blk < NBLK) {
+                    const T* src = kstage + (32 * st + 8 * beta + ((lane & 15) >> 2)) * kPitch +
+                                   16 * blk + 4 * (lane & 3);
+                    ktf[nb][st] = lds_frag_tr<T>(src, kPitch);
+                } else {
+                    u32x4_t z = {0u, 0u, 0u, 0u};
+                    ktf[nb][st] = __builtin_bit_cast(frag_t, z);
+                }
+            }
+        }
+        __syncthreads();
+    }
+
+    f32x16_t dk_acc[DV], dv_acc[DV];
+#pragma unroll
+    for (int x = 0; x < DV; ++x)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dk_acc[x][r] = 0.f, dv_acc[x][r] = 0.f;
+
+    int i_lo, i_hi;
+    query_range(a, k0, min(k0 + kBwdBN, a.sk), i_lo, i_hi);
+    const int t_lo = i_lo / kBwdBM;
+    const int t_hi = (i_hi + kBwdBM - 1) / kBwdBM;
+
+    // Per-lane bias when it does not depend on the query (the compact [B,1,1,Sk] layout).
+    const bool bias_per_key = a.has_bias && a.bs[2] == 0;
+    float bias_k = 0.f;
+    if (bias_per_key && key < a.sk)
+        bias_k = a.bias[b * a.bs[0] + h * a.bs[1] + (int64_t)key * a.bs[3]] * kLog2e;
+
+    QStage qst, gst;
+    float stat_reg = 0.f;
+    auto load_stats = [&](int i0) {
+        // threads 0..31 fetch lse (log2 domain, +inf for rows past the end so that P = 0),
+        // threads 32..63 fetch delta
+        if (threadIdx.x < 64) {
+            const int i = i0 + (threadIdx.x & 31);
+            if (threadIdx.x < 32)
+                stat_reg = i < a.sq ? lse_base[i] * kLog2e : INFINITY;
+            else
+                stat_reg = i < a.sq ? delta_base[i] : 0.f;
+        }
+    };
+    auto store_stats = [&](int buf) {
+        if (threadIdx.x < 64) stat_lds[buf * 64 + threadIdx.x] = stat_reg;
+    };
+
+    if (t_lo < t_hi) {
+        qst.load(q_base, a.qs[1], t_lo * kBwdBM, a.sq, a.d);
+        gst.load(g_base, a.os[1], t_lo * kBwdBM, a.sq, a.d);
+        load_stats(t_lo * kBwdBM);
+        qst.store(q_lds);
+        gst.store(g_lds);
+        store_stats(0);
+    }
+    __syncthreads();
+
+    for (int t = t_lo; t < t_hi; ++t) {
+        const int buf = (t - t_lo) & 1;
+        const T* qt = q_lds + buf * SM::kQTile;
+        const T* gt = g_lds + buf * SM::kQTile;
+        T* dst = ds_lds + buf * SM::kDsTile;
+        const float* lse_t = stat_lds + buf * 64;
+        const float* delta_t = lse_t + 32;
+        const int i0 = t * kBwdBM;
+        const bool have_next = t + 1 < t_hi;
+        if (have_next) {
+            qst.load(q_base, a.qs[1], i0 + kBwdBM, a.sq, a.d);
+            gst.load(g_base, a.os[1], i0 + kBwdBM, a.sq, a.d);
+            load_stats(i0 + kBwdBM);
+        }
+
+        const int i_last = min(i0 + kBwdBM, a.sq) - 1;
+        // wavefront-uniform activity of each 32-key slab of this workgroup for this query tile
+        auto slab_active = [&](int w) {
+            const int ks0 = k0 + 32 * w;
+            if (ks0 >= a.sk) return false;
+            if (a.causal && ks0 > i_last) return false;
+            if (a.window > 0 && i0 - (ks0 + 31) >= a.window) return false;
+            return true;
+        };
+        const bool active = slab_active(wave);
+
+        if (active) {
+            // ---- S = Q K^T, dP = dO V^T ----
+            f32x16_t s_acc, p_acc;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s_acc[r] = 0.f, p_acc[r] = 0.f;
+            {
+                const T* qrow = qt + pi_row(c_loc) * kPitch + 8 * g;
+                const T* grow = gt + pi_row(c_loc) * kPitch + 8 * g;
+#pragma unroll
+                for (int x = 0; x < DK; ++x) {
+                    s_acc = Mma<T>::mma32(lds_frag<T>(qrow + 16 * x), kf[x], s_acc);
+                    p_acc = Mma<T>::mma32(lds_frag<T>(grow + 16 * x), vf[x], p_acc);
+                }
+            }
+            const bool need_mask = (kw0 + 32 > a.sk) || (a.causal && kw0 + 31 > i0) ||
+                                   (a.window > 0 && i_last - kw0 >= a.window);
+            // ---- P and dS ----
+            uint32_t pw[8], dw[8];
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                const int qoff = acc_row(4 * r4, g);
+                const f32x4_t lse4 = *reinterpret_cast<const f32x4_t*>(lse_t + qoff);
+                const f32x4_t del4 = *reinterpret_cast<const f32x4_t*>(delta_t + qoff);
+                float pv[4], dv[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int i = i0 + qoff + e;
+                    float s = __builtin_fmaf(s_acc[4 * r4 + e], a.scale_log2, -lse4[e]);
+                    if (a.has_bias) {
+                        if (bias_per_key)
+                            s += bias_k;
+                        else if (i < a.sq && key < a.sk)
+                            s += a.bias[b * a.bs[0] + h * a.bs[1] + (int64_t)i * a.bs[2] +
+                                        (int64_t)key * a.bs[3]] * kLog2e;
+                    }
+                    float p = fast_exp2(s);
+                    if (need_mask && !key_visible(a, i, key)) p = 0.f;
+                    float dp = p_acc[4 * r4 + e];
+                    float pd = p;
+                    if (a.dropout) {
+                        float keep = 0.f;
+                        if (i < a.sq && key < a.sk) {
+                            const uint64_t el =
+                                ((uint64_t)bh * a.sq + (uint64_t)i) * (uint64_t)a.sk + (uint64_t)key;
+                            bool kb;
+                            if (a.dropout_fast)
+                                kb = (dropout_keep4(a.rng, el >> 2) >> (el & 3)) & 1u;
+                            else
+                                kb = dropout_keep1(a.rng, el);
+                            keep = kb ? a.rng.inv_keep : 0.f;
+                        }
+                        pd = p * keep;
+                        dp = dp * keep;
+                    }
+                    pv[e] = pd;
+                    dv[e] = p * (dp - del4[e]);
+                }
+                pw[2 * r4] = pack2<T>(pv[0], pv[1]);
+                pw[2 * r4 + 1] = pack2<T>(pv[2], pv[3]);
+                dw[2 * r4] = pack2<T>(dv[0], dv[1]);
+                dw[2 * r4 + 1] = pack2<T>(dv[2], dv[3]);
+                // dS^T slab for the dQ pass: row = key (local), columns = 4 consecutive queries
+                u32x2_t w2 = {dw[2 * r4], dw[2 * r4 + 1]};
+                *reinterpret_cast<u32x2_t*>(dst + (wave * 32 + c_loc) * kDsPitch + qoff) = w2;
+            }
+            // ---- dV^T += dO^T P,  dK^T += Q^T dS ----
+#pragma unroll
+            for (int hh = 0; hh < 2; ++hh) {
+                u32x4_t pq = {pw[4 * hh], pw[4 * hh + 1], pw[4 * hh + 2], pw[4 * hh + 3]};
+                u32x4_t dq4 = {dw[4 * hh], dw[4 * hh + 1], dw[4 * hh + 2], dw[4 * hh + 3]};
+                const frag_t pf = __builtin_bit_cast(frag_t, pq);
+                const frag_t df = __builtin_bit_cast(frag_t, dq4);
+                const int off = (16 * hh + 8 * g + ((lane & 15) >> 2)) * kPitch +
+                                ((lane >> 4) & 1) * 16 + 4 * (lane & 3);
+#pragma unroll
+                for (int x = 0; x < DV; ++x) {
+                    dv_acc[x] =
+                        Mma<T>::mma32(lds_frag_tr<T>(gt + off + 32 * x, kPitch), pf, dv_acc[x]);
+                    dk_acc[x] =
+                        Mma<T>::mma32(lds_frag_tr<T>(qt + off + 32 * x, kPitch), df, dk_acc[x]);
+                }
+            }
+        }
+
+        // stage the next query tile (its buffer was last read before the previous barrier)
+        if (have_next) {
+            qst.store(q_lds + (buf ^ 1) * SM::kQTile);
+            gst.store(g_lds + (buf ^ 1) * SM::kQTile);
+            store_stats(buf ^ 1);
+        }
+        __syncthreads();
+
+        // ---- dQ tile = dS K over all active key slabs of the workgroup ----
+        {
+            const int beta = lane >> 4;
+            const int n16 = lane & 15;
+#pragma unroll
+            for (int nb = 0; nb < NDB; ++nb) {
+                const int blk = wave + nb * kBwdWaves;
+                if (blk >= NBLK) continue;
+                f32x4_t acc[2];
+#pragma unroll
+                for (int qb = 0; qb < 2; ++qb) acc[qb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+                bool any = false;
+#pragma unroll
+                for (int st = 0; st < kBwdWaves; ++st) {
+                    if (!slab_active(st)) continue;
+                    any = true;
+                    const T* src =
+                        dst + (32 * st + 8 * beta + (n16 >> 2)) * kDsPitch + 4 * (lane & 3);
+#pragma unroll
+                    for (int qb = 0; qb < 2; ++qb)
+                        acc[qb] = Mma<T>::mma16(lds_frag_tr<T>(src + 16 * qb, kDsPitch),
+                                                ktf[nb][st], acc[qb]);
+                }
+                if (!any) continue;
+                const int dcol = 16 * blk + n16;
+                if (dcol < a.d) {
+#pragma unroll
+                    for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+                        for (int r = 0; r < 4; ++r) {
+                            const int i = i0 + 16 * qb + 4 * beta + r;
+                            if (i < a.sq)
+                                unsafeAtomicAdd(dq_base + (int64_t)i * a.d + dcol, acc[qb][r]);
+                        }
+                }
+            }
+        }
+    }
+
+    // ---- write dK, dV ----
+    if (key < a.sk) {
+        T* dk_row = reinterpret_cast<T*>(a.dk) + b * a.dks[0] + (int64_t)key * a.dks[1] + h * a.dks[2];
+        T* dv_row = reinterpret_cast<T*>(a.dv) + b * a.dvs[0] + (int64_t)key * a.dvs[1] + h * a.dvs[2];
+#pragma unroll
+        for (int x = 0; x < DV; ++x)
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                const int d0 = x * 32 + 8 * r4 + 4 * g;
+                if (d0 < a.d) {
+                    u32x2_t wk, wv;
+                    wk.x = pack2<T>(dk_acc[x][4 * r4] * a.scale, dk_acc[x][4 * r4 + 1] * a.scale);
+                    wk.y = pack2<T>(dk_acc[x][4 * r4 + 2] * a.scale, dk_acc[x][4 * r4 + 3] * a.scale);
+                    wv.x = pack2<T>(dv_acc[x][4 * r4], dv_acc[x][4 * r4 + 1]);
+                    wv.y = pack2<T>(dv_acc[x][4 * r4 + 2], dv_acc[x][4 * r4 + 3]);
+                    *reinterpret_cast<u32x2_t*>(dk_row + d0) = wk;
+                    *reinterpret_cast<u32x2_t*>(dv_row + d0) = wv;
+                }
+            }
+    }
+}
+
+template <typename T, int DPAD>
+int launch_bwd(const AttnArgs& a, hipStream_t st) {
+    typedef BwdSmem<T, DPAD> SM;
+    const size_t smem = SM::kBytes;
+    const int n_kt = (a.sk + kBwdBN - 1) / kBwdBN;
+    const int64_t blocks = (int64_t)n_kt * a.batch * a.heads;
+    if (blocks <= 0 || blocks > 0x7FFFFFFF) return SLAPO_ERR_SHAPE;
+    auto kern = attn_bwd_kernel<T, DPAD>;
+    if (smem > 48 * 1024) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)smem) != hipSuccess)
+            return SLAPO_ERR_LAUNCH;
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kBwdThreads), smem, st, a);
+    return check_launch();
+}
+
+template <typename T>
+int dispatch_bwd(const AttnArgs& a, hipStream_t st) {
+    if (a.d <= 32) return launch_bwd<T, 32>(a, st);
+    if (a.d <= 64) return launch_bwd<T, 64>(a, st);
+    if (a.d <= 96) return launch_bwd<T, 96>(a, st);
+    if (a.d <= 128) return launch_bwd<T, 128>(a, st);
+    return SLAPO_ERR_SHAPE;
+}
+
+}  // namespace
+
+namespace slapo {
+int attn_bwd_mfma(const AttnArgs& a, int dtype, hipStream_t st) {
+    if (dtype == SLAPO_F16) return dispatch_bwd<f16_t>(a, st);
+    if (dtype == SLAPO_BF16) return dispatch_bwd<bf16_t>(a, st);
+    return SLAPO_ERR_DTYPE;
+}
+}  // namespace slapo

@@ -1,0 +1,256 @@
+// C-ABI entry points of the attention path: argument validation, kernel selection (MFMA kernels
+// for fp16 / bf16, FMA kernels for fp32) and the small helper kernels around the backward
+// (delta = rowsum(dO * O), dQ accumulator clear and fp32 -> T conversion).
+#include "attn_common.h"
+
+namespace slapo {
+int attn_fwd_mfma(const AttnArgs& a, int dtype, hipStream_t st);
+int attn_bwd_mfma(const AttnArgs& a, int dtype, hipStream_t st);
+int attn_fwd_f32(const AttnArgs& a, hipStream_t st);
+int attn_bwd_f32(const AttnArgs& a, hipStream_t st);
+}  // namespace slapo
+
+using namespace slapo;
+
+namespace {
+
+// delta[bh, i] = sum_d dO[b,i,h,d] * O[b,i,h,d]; eight lanes share a row, 16 bytes per lane.
+template <typename T>
+__global__ __launch_bounds__(256) void attn_delta_kernel(const AttnArgs a) {
+    constexpr int V = Elem<T>::kPerVec;
+    const int64_t row = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 3;
+    const int sub = threadIdx.x & 7;
+    const int64_t n_rows = (int64_t)a.batch * a.heads * a.sq;
+    float acc = 0.f;
+    if (row < n_rows) {
+        const int i = (int)(row % a.sq);
+        const int bh = (int)(row / a.sq);
+        const int b = bh / a.heads, h = bh % a.heads;
+        const int64_t off = b * a.os[0] + (int64_t)i * a.os[1] + h * a.os[2];
+        const T* o = reinterpret_cast<const T*>(a.o) + off;
+        const T* g = reinterpret_cast<const T*>(a.dout) + off;
+        // head_dim is a multiple of V on this path (checked by the dispatcher)
+        for (int c = sub * V; c < a.d; c += 8 * V) {
+            const Packet<T> po = load_packet<T>(o + c);
+            const Packet<T> pg = load_packet<T>(g + c);
+#pragma unroll
+            for (int e = 0; e < V; ++e)
+                acc = __builtin_fmaf(Elem<T>::to_f32(po.v[e]), Elem<T>::to_f32(pg.v[e]), acc);
+        }
+    }
+    acc += __shfl_xor(acc, 1, 64);
+    acc += __shfl_xor(acc, 2, 64);
+    acc += __shfl_xor(acc, 4, 64);
+    if (row < n_rows && sub == 0) a.delta[row] = acc;
+}
+
+// Scalar variant for fp32 tensors whose rows are not 16-byte aligned.
+__global__ __launch_bounds__(256) void attn_delta_scalar_kernel(const AttnArgs a) {
+    const int64_t row = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t n_rows = (int64_t)a.batch * a.heads * a.sq;
+    if (row >= n_rows) return;
+    const int i = (int)(row % a.sq);
+    const int bh = (int)(row / a.sq);
+    const int b = bh / a.heads, h = bh % a.heads;
+    const int64_t off = b * a.os[0] + (int64_t)i * a.os[1] + h * a.os[2];
+    const float* o = reinterpret_cast<const float*>(a.o) + off;
+    const float* g = reinterpret_cast<const float*>(a.dout) + off;
+    float acc = 0.f;
+    for (int e = 0; e < a.d; ++e) acc = __builtin_fmaf(o[e], g[e], acc);
+    a.delta[row] = acc;
+}
+
+__global__ __launch_bounds__(256) void fill_zero_kernel(f32x4_t* p, int64_t n4) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n4) p[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+}
+
+// dq[b,i,h,:] = T(scale * dq_acc[bh,i,:]);  8 lanes per row, 4 floats per lane per trip.
+template <typename T>
+__global__ __launch_bounds__(256) void dq_convert_kernel(const AttnArgs a, const float* acc) {
+    const int64_t row = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 3;
+    const int sub = threadIdx.x & 7;
+    const int64_t n_rows = (int64_t)a.batch * a.heads * a.sq;
+    if (row >= n_rows) return;
+    const int i = (int)(row % a.sq);
+    const int bh = (int)(row / a.sq);
+    const int b = bh / a.heads, h = bh % a.heads;
+    T* out = reinterpret_cast<T*>(a.dq) + b * a.dqs[0] + (int64_t)i * a.dqs[1] + h * a.dqs[2];
+    const float* src = acc + row * a.d;
+    for (int c = sub * 4; c < a.d; c += 32) {
+        const f32x4_t v = *reinterpret_cast<const f32x4_t*>(src + c);
+        u32x2_t w;
+        w.x = pack2<T>(v.x * a.scale, v.y * a.scale);
+        w.y = pack2<T>(v.z * a.scale, v.w * a.scale);
+        *reinterpret_cast<u32x2_t*>(out + c) = w;
+    }
+}
+
+bool strides_ok(const int64_t s[3], int mult) {
+    return s[0] % mult == 0 && s[1] % mult == 0 && s[2] % mult == 0;
+}
+
+int fill_args(const slapo_attn_params* p, AttnArgs* a, bool backward) {
+    if (!p) return SLAPO_ERR_ARG;
+    if (p->batch <= 0 || p->heads <= 0 || p->seqlen_q <= 0 || p->seqlen_k <= 0 ||
+        p->head_dim <= 0)
+        return SLAPO_ERR_SHAPE;
+    if (p->head_dim > 128) return SLAPO_ERR_SHAPE;
+    if ((int64_t)p->batch * p->heads > 0x7FFFFFFF / 2) return SLAPO_ERR_SHAPE;
+    if (!(p->p_drop >= 0.f && p->p_drop <= 1.f)) return SLAPO_ERR_ARG;
+    if (p->window < 0) return SLAPO_ERR_ARG;
+    const bool half = p->dtype == SLAPO_F16 || p->dtype == SLAPO_BF16;
+    if (!half && p->dtype != SLAPO_F32) return SLAPO_ERR_DTYPE;
+    if (half) {
+        if (p->head_dim % 8 != 0) return SLAPO_ERR_SHAPE;
+        if (!strides_ok(p->q_strides, 8) || !strides_ok(p->k_strides, 8) ||
+            !strides_ok(p->v_strides, 8) || !strides_ok(p->o_strides, 8))
+            return SLAPO_ERR_ALIGN;
+    }
+    for (int i = 0; i < 3; ++i) {
+        a->qs[i] = p->q_strides[i];
+        a->ks[i] = p->k_strides[i];
+        a->vs[i] = p->v_strides[i];
+        a->os[i] = p->o_strides[i];
+    }
+    for (int i = 0; i < 4; ++i) a->bs[i] = p->bias_strides[i];
+    a->batch = p->batch;
+    a->heads = p->heads;
+    a->sq = p->seqlen_q;
+    a->sk = p->seqlen_k;
+    a->d = p->head_dim;
+    a->causal = p->causal ? 1 : 0;
+    a->window = p->window;
+    a->scale = p->scale;
+    a->scale_log2 = p->scale * kLog2e;
+    a->dropout = p->p_drop > 0.f ? 1 : 0;
+    a->dropout_fast = 0;
+    if (a->dropout) {
+        const int64_t numel = (int64_t)p->batch * p->heads * p->seqlen_q * p->seqlen_k;
+        if (!plan_ok(&p->plan, numel)) return SLAPO_ERR_ARG;
+        a->rng = make_dropout_state(p->plan, (double)p->p_drop, p->seed, p->offset);
+        a->dropout_fast = (p->plan.vec >= 4 && p->seqlen_k % 4 == 0) ? 1 : 0;
+    } else {
+        a->rng = DropoutState{};
+    }
+    (void)backward;
+    return SLAPO_OK;
+}
+
+void set_bias(AttnArgs* a, const float* bias) {
+    a->bias = bias;
+    a->has_bias = bias ? 1 : 0;
+    a->bias_vec4 = 0;
+    if (bias && a->bs[3] == 1 && a->bs[2] == 0 && aligned16(bias) && a->bs[0] % 4 == 0 &&
+        a->bs[1] % 4 == 0)
+        a->bias_vec4 = 1;
+}
+
+bool half_ptrs_ok(std::initializer_list<const void*> ptrs) {
+    for (const void* p : ptrs)
+        if (!p || !aligned16(p)) return false;
+    return true;
+}
+
+}  // namespace
+
+extern "C" int slapo_amd_attn_fwd(const slapo_attn_params* prm, const void* q, const void* k,
+                                  const void* v, const float* bias, void* o, float* lse,
+                                  void* stream) {
+    AttnArgs a = {};
+    int rc = fill_args(prm, &a, false);
+    if (rc != SLAPO_OK) return rc;
+    if (!q || !k || !v || !o || !lse) return SLAPO_ERR_ARG;
+    a.q = q, a.k = k, a.v = v, a.o = o, a.lse = lse;
+    set_bias(&a, bias);
+    hipStream_t st = (hipStream_t)stream;
+    if (prm->dtype == SLAPO_F32) return attn_fwd_f32(a, st);
+    if (!half_ptrs_ok({q, k, v, o})) return SLAPO_ERR_ALIGN;
+    return attn_fwd_mfma(a, prm->dtype, st);
+}
+
+extern "C" size_t slapo_amd_attn_bwd_workspace_bytes(const slapo_attn_params* prm) {
+    if (!prm || prm->batch <= 0 || prm->heads <= 0 || prm->seqlen_q <= 0 || prm->head_dim <= 0)
+        return 0;
+    const size_t rows = (size_t)prm->batch * prm->heads * prm->seqlen_q;
+    size_t bytes = rows * sizeof(float);  // delta
+    if (prm->dtype != SLAPO_F32) bytes += rows * (size_t)prm->head_dim * sizeof(float);  // dQ acc
+    return bytes;
+}
+
+extern "C" int slapo_amd_attn_bwd(const slapo_attn_params* prm, const void* q, const void* k,
+                                  const void* v, const float* bias, const void* o,
+                                  const void* dout, const float* lse, void* dq, void* dk,
+                                  void* dv, const int64_t dq_strides[3],
+                                  const int64_t dk_strides[3], const int64_t dv_strides[3],
+                                  void* workspace, size_t workspace_bytes, void* stream) {
+    AttnArgs a = {};
+    int rc = fill_args(prm, &a, true);
+    if (rc != SLAPO_OK) return rc;
+    if (!q || !k || !v || !o || !dout || !lse || !dq || !dk || !dv || !dq_strides ||
+        !dk_strides || !dv_strides)
+        return SLAPO_ERR_ARG;
+    if (!workspace || workspace_bytes < slapo_amd_attn_bwd_workspace_bytes(prm) ||
+        !aligned16(workspace))
+        return SLAPO_ERR_WORKSPACE;
+    for (int i = 0; i < 3; ++i) {
+        a.dqs[i] = dq_strides[i];
+        a.dks[i] = dk_strides[i];
+        a.dvs[i] = dv_strides[i];
+    }
+    a.q = q, a.k = k, a.v = v, a.o = const_cast<void*>(o), a.dout = dout;
+    a.lse = const_cast<float*>(lse);
+    a.dk = dk, a.dv = dv;
+    set_bias(&a, bias);
+    hipStream_t st = (hipStream_t)stream;
+
+    const int64_t rows = (int64_t)a.batch * a.heads * a.sq;
+    const bool is_f32 = prm->dtype == SLAPO_F32;
+    // workspace: [dQ accumulator (16-bit types only)] [delta]
+    float* dq_acc = reinterpret_cast<float*>(workspace);
+    a.delta = is_f32 ? dq_acc : dq_acc + rows * a.d;
+
+    if (is_f32) {
+        const bool vec_ok = a.d % 4 == 0 && aligned16(o) && aligned16(dout) &&
+                            strides_ok(prm->o_strides, 4);
+        if (vec_ok) {
+            const unsigned blocks = (unsigned)((rows * 8 + 255) / 256);
+            hipLaunchKernelGGL((attn_delta_kernel<float>), dim3(blocks), dim3(256), 0, st, a);
+        } else {
+            const unsigned blocks = (unsigned)((rows + 255) / 256);
+            hipLaunchKernelGGL(attn_delta_scalar_kernel, dim3(blocks), dim3(256), 0, st, a);
+        }
+        rc = check_launch();
+        if (rc != SLAPO_OK) return rc;
+        a.dq = dq;
+        return attn_bwd_f32(a, st);
+    }
+
+    if (!half_ptrs_ok({q, k, v, o, dout, dq, dk, dv})) return SLAPO_ERR_ALIGN;
+    if (!strides_ok(dq_strides, 8) || !strides_ok(dk_strides, 8) || !strides_ok(dv_strides, 8))
+        return SLAPO_ERR_ALIGN;
+
+    const unsigned row_blocks = (unsigned)((rows * 8 + 255) / 256);
+    if (prm->dtype == SLAPO_F16)
+        hipLaunchKernelGGL((attn_delta_kernel<f16_t>), dim3(row_blocks), dim3(256), 0, st, a);
+    else
+        hipLaunchKernelGGL((attn_delta_kernel<bf16_t>), dim3(row_blocks), dim3(256), 0, st, a);
+    const int64_t n4 = rows * a.d / 4;  // head_dim % 8 == 0
+    hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, st,
+                       reinterpret_cast<f32x4_t*>(dq_acc), n4);
+    rc = check_launch();
+    if (rc != SLAPO_OK) return rc;
+
+    a.dq = dq_acc;
+    rc = attn_bwd_mfma(a, prm->dtype, st);
+    if (rc != SLAPO_OK) return rc;
+
+    a.dq = dq;
+    if (prm->dtype == SLAPO_F16)
+        hipLaunchKernelGGL((dq_convert_kernel<f16_t>), dim3(row_blocks), dim3(256), 0, st, a,
+                           dq_acc);
+    else
+        hipLaunchKernelGGL((dq_convert_kernel<bf16_t>), dim3(row_blocks), dim3(256), 0, st, a,
+                           dq_acc);
+    return check_launch();
+}

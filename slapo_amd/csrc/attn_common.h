@@ -1,0 +1,171 @@
+// Pieces shared by the attention kernels: MFMA wrappers for fp16/bf16 on gfx950, the LDS
+// transpose read, tile staging (global -> registers -> LDS), masks and the kernel argument block.
+//
+// MFMA v_mfma_f32_32x32x16_{f16,bf16} (one wavefront, lane l, g = l / 32):
+//   A operand: lane holds row (l % 32), 8 consecutive k-slots of lane-group g;
+//   B operand: lane holds column (l % 32), the same 8 k-slots;
+//   C/D:       register r of lane l is element (row 8*(r/4) + 4*g + r%4, column l % 32).
+// The k-slot <-> data mapping is free as long as A and B agree, and the row <-> data mapping of
+// the A operand is free as well; both freedoms are used below to keep every fragment a plain
+// 128-bit LDS read or two transposing 64-bit reads.
+#pragma once
+#include "common.h"
+
+namespace slapo {
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+template <typename T>
+struct Mma;
+
+template <>
+struct Mma<f16_t> {
+    typedef f16x8_t frag;
+    typedef f16x4_t half_frag;
+    static __device__ __forceinline__ f32x16_t mma32(frag a, frag b, f32x16_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ f32x4_t mma16(frag a, frag b, f32x4_t c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+    }
+};
+template <>
+struct Mma<bf16_t> {
+    typedef bf16x8_t frag;
+    typedef bf16x4_t half_frag;
+    static __device__ __forceinline__ f32x16_t mma32(frag a, frag b, f32x16_t c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+    static __device__ __forceinline__ f32x4_t mma16(frag a, frag b, f32x4_t c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+    }
+};
+
+typedef short i16x4_t __attribute__((ext_vector_type(4)));
+
+// LDS transpose read (ds_read_b64_tr_b16).  Within each block of 16 lanes, lane n receives
+// element e = 0..3 from source lane (4*e + n/4), 16-bit word (n % 4) of that lane's 8 bytes.
+// With source lane i pointing at row (i/4), columns 4*(i%4).. of a row-major tile, lane n gets
+// the four rows of column n: a 4x16 -> 16x4 transpose.
+__device__ __forceinline__ u32x2_t lds_read_tr16(const void* lds_ptr) {
+    i16x4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16(
+        (i16x4_t __attribute__((address_space(3)))*)(uintptr_t)(
+            (uint32_t)(uintptr_t)lds_ptr));
+    return __builtin_bit_cast(u32x2_t, v);
+}
+
+// Fragment made of two transposing reads: slots 0..3 from rows r0..r0+3, slots 4..7 from
+// r0+4..r0+7 of a row-major LDS tile with `pitch` elements per row.
+template <typename T>
+__device__ __forceinline__ typename Mma<T>::frag lds_frag_tr(const T* tile, int pitch) {
+    const u32x2_t lo = lds_read_tr16(tile);
+    const u32x2_t hi = lds_read_tr16(tile + 4 * pitch);
+    u32x4_t v = {lo.x, lo.y, hi.x, hi.y};
+    return __builtin_bit_cast(typename Mma<T>::frag, v);
+}
+
+template <typename T>
+__device__ __forceinline__ typename Mma<T>::frag lds_frag(const T* p) {
+    return *reinterpret_cast<const typename Mma<T>::frag*>(p);
+}
+
+// Row permutation applied when a 32-row A operand is gathered: MFMA row rho takes data row
+// pi(rho), pi = swap of bits 2 and 3.  With it, accumulator registers 8*h .. 8*h+7 of lane-group
+// g hold the eight CONSECUTIVE data rows 16*h + 8*g .. +7, i.e. they form, in order, the k-slots
+// of a B operand for the next MFMA.
+__device__ __forceinline__ int pi_row(int rho) {
+    return (rho & ~0xC) | ((rho & 4) << 1) | ((rho & 8) >> 1);
+}
+// Data row (0..31) held by accumulator register r of lane-group g under that permutation.
+__device__ __forceinline__ constexpr int acc_row(int r, int g) {
+    return ((r >> 3) << 4) + (g << 3) + (((r >> 2) & 1) << 2) + (r & 3);
+}
+
+template <typename T>
+__device__ __forceinline__ uint32_t pack2(float a, float b) {
+    typedef T pair_t __attribute__((ext_vector_type(2)));
+    pair_t p = {(T)a, (T)b};
+    return __builtin_bit_cast(uint32_t, p);
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+__device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32, 64); }
+
+// Kernel argument block (filled by the host dispatcher from slapo_attn_params).
+struct AttnArgs {
+    const void* q;
+    const void* k;
+    const void* v;
+    void* o;
+    const void* dout;
+    void* dq;  // fp32 accumulator in the MFMA backward, element type T in the fp32 kernels
+    void* dk;
+    void* dv;
+    const float* bias;
+    float* lse;
+    float* delta;
+    int64_t qs[3], ks[3], vs[3], os[3], dqs[3], dks[3], dvs[3];
+    int64_t bs[4];
+    int batch, heads, sq, sk, d;
+    int causal, window;
+    int has_bias, bias_vec4;  // bias_vec4: s3 == 1, s2 == 0 rows 16B-aligned
+    int dropout, dropout_fast;  // dropout_fast: plan.vec >= 4 and sk % 4 == 0
+    float scale, scale_log2;
+    DropoutState rng;
+};
+
+__device__ __forceinline__ bool key_visible(const AttnArgs& a, int i, int j) {
+    return j < a.sk && (!a.causal || j <= i) && (a.window <= 0 || i - j < a.window);
+}
+
+// First / one-past-last key that any query in [q_lo, q_hi) may see.
+__device__ __forceinline__ void key_range(const AttnArgs& a, int q_lo, int q_hi, int& j_lo,
+                                          int& j_hi) {
+    j_hi = a.causal ? min(a.sk, q_hi) : a.sk;
+    j_lo = a.window > 0 ? max(0, q_lo - a.window + 1) : 0;
+}
+// First / one-past-last query that can see any key in [k_lo, k_hi).
+__device__ __forceinline__ void query_range(const AttnArgs& a, int k_lo, int k_hi, int& i_lo,
+                                            int& i_hi) {
+    i_lo = a.causal ? min(k_lo, a.sq) : 0;
+    i_hi = a.window > 0 ? min(a.sq, k_hi - 1 + a.window) : a.sq;
+}
+
+// Stage a [64 x DPAD] tile of T (rows row0.., zero beyond n_rows / beyond d) through registers.
+template <typename T, int DPAD, int ROWS, int THREADS>
+struct TileStage {
+    static constexpr int kChunksPerRow = DPAD / 8;
+    static constexpr int kChunks = ROWS * kChunksPerRow;
+    static constexpr int kPerThread = (kChunks + THREADS - 1) / THREADS;
+    static constexpr int kPitch = DPAD + 8;
+    u32x4_t r[kPerThread];
+
+    __device__ __forceinline__ void load(const T* base, int64_t row_stride, int row0, int n_rows,
+                                         int d) {
+#pragma unroll
+        for (int u = 0; u < kPerThread; ++u) {
+            const int c = threadIdx.x + u * THREADS;
+            const int row = c / kChunksPerRow;
+            const int cc = c % kChunksPerRow;
+            const int gr = row0 + row;
+            u32x4_t v = {0u, 0u, 0u, 0u};
+            if ((kChunks % THREADS == 0 || c < kChunks) && gr < n_rows && cc * 8 < d)
+                v = *reinterpret_cast<const u32x4_t*>(base + (int64_t)gr * row_stride + cc * 8);
+            r[u] = v;
+        }
+    }
+    __device__ __forceinline__ void store(T* lds) const {
+#pragma unroll
+        for (int u = 0; u < kPerThread; ++u) {
+            const int c = threadIdx.x + u * THREADS;
+            if (kChunks % THREADS != 0 && c >= kChunks) continue;
+            const int row = c / kChunksPerRow;
+            const int cc = c % kChunksPerRow;
+            *reinterpret_cast<u32x4_t*>(lds + row * kPitch + cc * 8) = r[u];
+        }
+    }
+};
+
+}  // namespace slapo

@@ -1,0 +1,514 @@
+// FusedMLP epilogues for gfx950: bias+GeLU(tanh) and bias+dropout(+residual), forward and
+// backward.  All four are single-pass, HBM-bound streaming kernels: every tensor element is
+// read or written exactly once through 128-bit accesses; the dropout mask is never stored
+// (it is regenerated from the Philox state), and the bias gradient is a deterministic two-stage
+// column reduction (per-block fp32 partials, then a tiny finishing kernel) -- no atomics.
+//
+// Formulas follow slapo/op/fused_bias.py:18-34 (bias_gelu / bias_gelu_back) and :67-74
+// (bias_dropout); math is fp32 inside, storage in the tensor dtype.
+#include "common.h"
+
+using namespace slapo;
+
+namespace {
+
+// gelu_tanh(x) = 0.5 x (1 + tanh(a)) with a = 0.79788456 x (1 + 0.044715 x^2)
+//             = x * sigma(2a),   sigma(z) = 1 / (1 + exp(-z)).
+// exp(-2a) = exp2(x * (K1 + K2 x^2)),  K1 = -2 log2(e) 0.79788456,  K2 = K1 * 0.044715.
+constexpr float kGeluK1 = -2.0f * 1.4426950408889634f * 0.79788456f;
+constexpr float kGeluK2 = kGeluK1 * 0.044715f;
+
+__device__ __forceinline__ float sigma2a(float x) {
+    const float t = x * x;
+    const float e = __builtin_amdgcn_exp2f(x * __builtin_fmaf(t, kGeluK2, kGeluK1));
+    return __builtin_amdgcn_rcpf(1.0f + e);
+}
+
+__device__ __forceinline__ float gelu_fwd(float x) { return x * sigma2a(x); }
+
+// d/dx: with t = tanh(a) = 2 s - 1:  0.5 (1 + t) = s,  1 - t^2 = 4 s (1 - s), so
+// ff = 0.5 x (1 - t^2)(0.79788456 + 0.1070322243 x^2) + 0.5 (1 + t)
+//    = s + 2 x s (1 - s)(0.79788456 + 0.1070322243 x^2).
+__device__ __forceinline__ float gelu_grad(float x) {
+    const float s = sigma2a(x);
+    const float poly = __builtin_fmaf(x * x, 0.1070322243f, 0.79788456f);
+    return __builtin_fmaf(2.0f * x * s * (1.0f - s), poly, s);
+}
+
+// V consecutive elements of T: V == Elem<T>::kPerVec uses one 128-bit access, V == 1 scalar.
+template <typename T, int V>
+struct Chunk {
+    T v[V];
+};
+
+template <typename T, int V>
+__device__ __forceinline__ Chunk<T, V> load_chunk(const T* p) {
+    Chunk<T, V> c;
+    if constexpr (V == 1) {
+        c.v[0] = *p;
+    } else {
+        static_assert(sizeof(Chunk<T, V>) == 16, "vector chunk must be 16 bytes");
+        *reinterpret_cast<u32x4_t*>(&c) =
+            __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(p));
+    }
+    return c;
+}
+template <typename T, int V>
+__device__ __forceinline__ Chunk<T, V> load_chunk_cached(const T* p) {
+    Chunk<T, V> c;
+    if constexpr (V == 1) {
+        c.v[0] = *p;
+    } else {
+        *reinterpret_cast<u32x4_t*>(&c) = *reinterpret_cast<const u32x4_t*>(p);
+    }
+    return c;
+}
+template <typename T, int V>
+__device__ __forceinline__ void store_chunk(T* p, const Chunk<T, V>& c) {
+    if constexpr (V == 1) {
+        *p = c.v[0];
+    } else {
+        __builtin_nontemporal_store(*reinterpret_cast<const u32x4_t*>(&c),
+                                    reinterpret_cast<u32x4_t*>(p));
+    }
+}
+
+// Keep-bits for V consecutive elements starting at element index e0 (e0 % V == 0).
+template <int V>
+__device__ __forceinline__ uint32_t keep_bits(const DropoutState& s, uint64_t e0) {
+    uint32_t bits = 0;
+    if constexpr (V % 4 == 0) {
+        if (s.vec >= 4) {
+#pragma unroll
+            for (int g = 0; g < V / 4; ++g) bits |= dropout_keep4(s, e0 / 4 + g) << (4 * g);
+            return bits;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < V; ++i) bits |= (dropout_keep1(s, e0 + i) ? 1u : 0u) << i;
+    return bits;
+}
+
+// ----------------------------------------------------------------------------------------
+// Forward kernels: flat over chunks; a block covers kUnroll * 256 consecutive chunks.
+// ----------------------------------------------------------------------------------------
+constexpr int kUnroll = 4;
+
+template <typename T, int V>
+__global__ __launch_bounds__(256) void bias_gelu_fwd_kernel(const T* __restrict__ y,
+                                                            const T* __restrict__ bias,
+                                                            T* __restrict__ out,
+                                                            uint64_t n_chunks,
+                                                            uint32_t chunks_per_row,
+                                                            uint32_t row_mask) {
+    const uint64_t base = (uint64_t)blockIdx.x * (256 * kUnroll) + threadIdx.x;
+    Chunk<T, V> in[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+        const uint64_t c = base + (uint64_t)u * 256;
+        if (c < n_chunks) in[u] = load_chunk<T, V>(y + c * V);
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+        const uint64_t c = base + (uint64_t)u * 256;
+        if (c >= n_chunks) continue;
+        const uint32_t col =
+            row_mask ? ((uint32_t)c & row_mask) : (uint32_t)(c % chunks_per_row);
+        const Chunk<T, V> b = load_chunk_cached<T, V>(bias + (uint64_t)col * V);
+        Chunk<T, V> o;
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+            const float x = Elem<T>::to_f32(in[u].v[i]) + Elem<T>::to_f32(b.v[i]);
+            o.v[i] = Elem<T>::from_f32(gelu_fwd(x));
+        }
+        store_chunk<T, V>(out + c * V, o);
+    }
+}
+
+template <typename T, int V, bool kResidual, bool kDropout>
+__global__ __launch_bounds__(256) void bias_dropout_residual_fwd_kernel(
+    const T* __restrict__ x, const T* __restrict__ bias, const T* __restrict__ residual,
+    T* __restrict__ out, uint64_t n_chunks, uint32_t chunks_per_row, uint32_t row_mask,
+    DropoutState s) {
+    const uint64_t base = (uint64_t)blockIdx.x * (256 * kUnroll) + threadIdx.x;
+    Chunk<T, V> in[kUnroll];
+    Chunk<T, V> res[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+        const uint64_t c = base + (uint64_t)u * 256;
+        if (c < n_chunks) {
+            in[u] = load_chunk<T, V>(x + c * V);
+            if constexpr (kResidual) res[u] = load_chunk<T, V>(residual + c * V);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < kUnroll; ++u) {
+        const uint64_t c = base + (uint64_t)u * 256;
+        if (c >= n_chunks) continue;
+        const uint32_t col =
+            row_mask ? ((uint32_t)c & row_mask) : (uint32_t)(c % chunks_per_row);
+        const Chunk<T, V> b = load_chunk_cached<T, V>(bias + (uint64_t)col * V);
+        uint32_t bits = 0xFFFFFFFFu;
+        if constexpr (kDropout) bits = keep_bits<V>(s, c * V);
+        Chunk<T, V> o;
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+            float v = Elem<T>::to_f32(in[u].v[i]) + Elem<T>::to_f32(b.v[i]);
+            if constexpr (kDropout) v = ((bits >> i) & 1u) ? v * s.inv_keep : 0.0f;
+            if constexpr (kResidual) v += Elem<T>::to_f32(res[u].v[i]);
+            o.v[i] = Elem<T>::from_f32(v);
+        }
+        store_chunk<T, V>(out + c * V, o);
+    }
+}
+
+// ----------------------------------------------------------------------------------------
+// Backward kernels: a block is 64 column-chunks x 4 row-lanes and walks kRowsPerBlock rows,
+// keeping per-thread fp32 column sums; the 4 row-lanes are combined through LDS and written
+// as one fp32 partial row per block.
+// ----------------------------------------------------------------------------------------
+constexpr int kRowsPerBlock = 64;
+constexpr int kRowLanes = 4;
+constexpr int kColLanes = 64;
+
+template <typename T, int V, typename F>
+__device__ __forceinline__ void colsum_walk(int64_t rows, int64_t cols, float* __restrict__ partial,
+                                            bool want_sum, F&& body) {
+    const int cx = threadIdx.x % kColLanes;
+    const int ry = threadIdx.x / kColLanes;
+    const int64_t chunk_col = (int64_t)blockIdx.x * kColLanes + cx;
+    const int64_t col0 = chunk_col * V;
+    const bool active = col0 < cols;
+    float acc[V];
+#pragma unroll
+    for (int i = 0; i < V; ++i) acc[i] = 0.f;
+    const int64_t r_begin = (int64_t)blockIdx.y * kRowsPerBlock;
+    if (active) {
+#pragma unroll 4
+        for (int it = 0; it < kRowsPerBlock / kRowLanes; ++it) {
+            const int64_t r = r_begin + ry + (int64_t)it * kRowLanes;
+            if (r < rows) body(r, col0, acc);
+        }
+    }
+    if (!want_sum) return;
+    __shared__ float red[kRowLanes][kColLanes][V + 1];
+#pragma unroll
+    for (int i = 0; i < V; ++i) red[ry][cx][i] = acc[i];
+    __syncthreads();
+    if (ry == 0 && active) {
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+            float t = red[0][cx][i];
+#pragma unroll
+            for (int k = 1; k < kRowLanes; ++k) t += red[k][cx][i];
+            partial[(int64_t)blockIdx.y * cols + col0 + i] = t;
+        }
+    }
+}
+
+template <typename T, int V>
+__global__ __launch_bounds__(256) void bias_gelu_bwd_kernel(const T* __restrict__ grad,
+                                                            const T* __restrict__ y,
+                                                            const T* __restrict__ bias,
+                                                            T* __restrict__ dx,
+                                                            float* __restrict__ partial,
+                                                            int64_t rows, int64_t cols,
+                                                            int want_sum) {
+    Chunk<T, V> b;
+    {
+        const int64_t col0 = ((int64_t)blockIdx.x * kColLanes + threadIdx.x % kColLanes) * V;
+        if (col0 < cols) b = load_chunk_cached<T, V>(bias + col0);
+    }
+    colsum_walk<T, V>(rows, cols, partial, want_sum != 0,
+                      [&](int64_t r, int64_t col0, float* acc) {
+                          const int64_t off = r * cols + col0;
+                          const Chunk<T, V> g = load_chunk<T, V>(grad + off);
+                          const Chunk<T, V> yy = load_chunk<T, V>(y + off);
+                          Chunk<T, V> o;
+#pragma unroll
+                          for (int i = 0; i < V; ++i) {
+                              const float x =
+                                  Elem<T>::to_f32(yy.v[i]) + Elem<T>::to_f32(b.v[i]);
+                              const float d = gelu_grad(x) * Elem<T>::to_f32(g.v[i]);
+                              o.v[i] = Elem<T>::from_f32(d);
+                              acc[i] += d;
+                          }
+                          store_chunk<T, V>(dx + off, o);
+                      });
+}
+
+template <typename T, int V, bool kDropout>
+__global__ __launch_bounds__(256) void bias_dropout_bwd_kernel(const T* __restrict__ grad,
+                                                               T* __restrict__ dx,
+                                                               float* __restrict__ partial,
+                                                               int64_t rows, int64_t cols,
+                                                               int want_sum, int write_dx,
+                                                               DropoutState s) {
+    colsum_walk<T, V>(rows, cols, partial, want_sum != 0,
+                      [&](int64_t r, int64_t col0, float* acc) {
+                          const int64_t off = r * cols + col0;
+                          const Chunk<T, V> g = load_chunk<T, V>(grad + off);
+                          uint32_t bits = 0xFFFFFFFFu;
+                          if constexpr (kDropout) bits = keep_bits<V>(s, (uint64_t)off);
+                          Chunk<T, V> o;
+#pragma unroll
+                          for (int i = 0; i < V; ++i) {
+                              float d = Elem<T>::to_f32(g.v[i]);
+                              if constexpr (kDropout)
+                                  d = ((bits >> i) & 1u) ? d * s.inv_keep : 0.0f;
+                              o.v[i] = Elem<T>::from_f32(d);
+                              acc[i] += d;
+                          }
+                          if (write_dx) store_chunk<T, V>(dx + off, o);
+                      });
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void colsum_finish_kernel(const float* __restrict__ partial,
+                                                            T* __restrict__ dbias,
+                                                            int64_t n_partials, int64_t cols) {
+    const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= cols) return;
+    float t = 0.f;
+    for (int64_t k = 0; k < n_partials; ++k) t += partial[k * cols + c];
+    dbias[c] = Elem<T>::from_f32(t);
+}
+
+// ----------------------------------------------------------------------------------------
+// Host dispatch
+// ----------------------------------------------------------------------------------------
+struct RowGeom {
+    uint64_t n_chunks;
+    uint32_t chunks_per_row;
+    uint32_t row_mask;
+    unsigned blocks;
+};
+
+inline bool flat_geom(int64_t rows, int64_t cols, int v, RowGeom* g) {
+    const int64_t cpr = cols / v;
+    if (cpr > 0x7FFFFFFF) return false;
+    g->chunks_per_row = (uint32_t)cpr;
+    g->n_chunks = (uint64_t)rows * (uint64_t)cpr;
+    g->row_mask = (cpr & (cpr - 1)) == 0 ? (uint32_t)(cpr - 1) : 0u;
+    if (cpr == 1) g->row_mask = 0;  // mask 0 means "use modulo"; modulo by 1 is fine
+    const uint64_t per_block = 256ull * kUnroll;
+    const uint64_t blocks = (g->n_chunks + per_block - 1) / per_block;
+    if (blocks > 0x7FFFFFFFull) return false;
+    g->blocks = (unsigned)blocks;
+    return true;
+}
+
+template <typename T>
+inline bool vector_ok(int64_t cols, std::initializer_list<const void*> ptrs) {
+    if (cols % Elem<T>::kPerVec != 0) return false;
+    for (const void* p : ptrs)
+        if (p && !aligned16(p)) return false;
+    return true;
+}
+
+template <typename T>
+int gelu_fwd_dispatch(const void* y, const void* bias, void* out, int64_t rows, int64_t cols,
+                      hipStream_t st) {
+    RowGeom g;
+    if (vector_ok<T>(cols, {y, bias, out})) {
+        constexpr int V = Elem<T>::kPerVec;
+        if (!flat_geom(rows, cols, V, &g)) return SLAPO_ERR_SHAPE;
+        hipLaunchKernelGGL((bias_gelu_fwd_kernel<T, V>), dim3(g.blocks), dim3(256), 0, st,
+                           (const T*)y, (const T*)bias, (T*)out, g.n_chunks, g.chunks_per_row,
+                           g.row_mask);
+    } else {
+        if (!flat_geom(rows, cols, 1, &g)) return SLAPO_ERR_SHAPE;
+        hipLaunchKernelGGL((bias_gelu_fwd_kernel<T, 1>), dim3(g.blocks), dim3(256), 0, st,
+                           (const T*)y, (const T*)bias, (T*)out, g.n_chunks, g.chunks_per_row,
+                           g.row_mask);
+    }
+    return check_launch();
+}
+
+template <typename T, int V>
+int dropres_fwd_launch(const void* x, const void* bias, const void* residual, void* out,
+                       int64_t rows, int64_t cols, bool dropout, const DropoutState& s,
+                       hipStream_t st) {
+    RowGeom g;
+    if (!flat_geom(rows, cols, V, &g)) return SLAPO_ERR_SHAPE;
+#define SLAPO_LAUNCH_DR(RES, DROP)                                                             \
+    hipLaunchKernelGGL((bias_dropout_residual_fwd_kernel<T, V, RES, DROP>), dim3(g.blocks),    \
+                       dim3(256), 0, st, (const T*)x, (const T*)bias, (const T*)residual,      \
+                       (T*)out, g.n_chunks, g.chunks_per_row, g.row_mask, s)
+    if (residual) {
+        if (dropout)
+            SLAPO_LAUNCH_DR(true, true);
+        else
+            SLAPO_LAUNCH_DR(true, false);
+    } else {
+        if (dropout)
+            SLAPO_LAUNCH_DR(false, true);
+        else
+            SLAPO_LAUNCH_DR(false, false);
+    }
+#undef SLAPO_LAUNCH_DR
+    return check_launch();
+}
+
+inline bool bwd_grid(int64_t rows, int64_t cols, int v, dim3* grid) {
+    const int64_t chunk_cols = (cols + v - 1) / v;
+    const int64_t gx = (chunk_cols + kColLanes - 1) / kColLanes;
+    const int64_t gy = (rows + kRowsPerBlock - 1) / kRowsPerBlock;
+    if (gx > 0x7FFFFFFF || gy > 65535) return false;
+    *grid = dim3((unsigned)gx, (unsigned)gy);
+    return true;
+}
+
+template <typename T>
+int finish_colsum(const float* partial, void* dbias, int64_t rows, int64_t cols, hipStream_t st) {
+    const int64_t n_partials = (rows + kRowsPerBlock - 1) / kRowsPerBlock;
+    const unsigned blocks = (unsigned)((cols + 255) / 256);
+    hipLaunchKernelGGL((colsum_finish_kernel<T>), dim3(blocks), dim3(256), 0, st, partial,
+                       (T*)dbias, n_partials, cols);
+    return check_launch();
+}
+
+template <typename T>
+int gelu_bwd_dispatch(const void* grad, const void* y, const void* bias, void* dx, void* dbias,
+                      void* ws, int64_t rows, int64_t cols, hipStream_t st) {
+    dim3 grid;
+    const int want = dbias ? 1 : 0;
+    if (vector_ok<T>(cols, {grad, y, bias, dx})) {
+        constexpr int V = Elem<T>::kPerVec;
+        if (!bwd_grid(rows, cols, V, &grid)) return SLAPO_ERR_SHAPE;
+        hipLaunchKernelGGL((bias_gelu_bwd_kernel<T, V>), grid, dim3(256), 0, st, (const T*)grad,
+                           (const T*)y, (const T*)bias, (T*)dx, (float*)ws, rows, cols, want);
+    } else {
+        if (!bwd_grid(rows, cols, 1, &grid)) return SLAPO_ERR_SHAPE;
+        hipLaunchKernelGGL((bias_gelu_bwd_kernel<T, 1>), grid, dim3(256), 0, st, (const T*)grad,
+                           (const T*)y, (const T*)bias, (T*)dx, (float*)ws, rows, cols, want);
+    }
+    int rc = check_launch();
+    if (rc != SLAPO_OK || !dbias) return rc;
+    return finish_colsum<T>((const float*)ws, dbias, rows, cols, st);
+}
+
+template <typename T, int V>
+int dropres_bwd_launch(const void* grad, void* dx, void* ws, int64_t rows, int64_t cols,
+                       bool dropout, int want, const DropoutState& s, hipStream_t st) {
+    dim3 grid;
+    if (!bwd_grid(rows, cols, V, &grid)) return SLAPO_ERR_SHAPE;
+    const int write_dx = dx ? 1 : 0;
+    if (dropout)
+        hipLaunchKernelGGL((bias_dropout_bwd_kernel<T, V, true>), grid, dim3(256), 0, st,
+                           (const T*)grad, (T*)dx, (float*)ws, rows, cols, want, write_dx, s);
+    else
+        hipLaunchKernelGGL((bias_dropout_bwd_kernel<T, V, false>), grid, dim3(256), 0, st,
+                           (const T*)grad, (T*)dx, (float*)ws, rows, cols, want, write_dx, s);
+    return check_launch();
+}
+
+template <typename T>
+int dropres_fwd_dispatch(const void* x, const void* bias, const void* residual, void* out,
+                         int64_t rows, int64_t cols, bool dropout, const DropoutState& s,
+                         hipStream_t st) {
+    if (vector_ok<T>(cols, {x, bias, residual, out}))
+        return dropres_fwd_launch<T, Elem<T>::kPerVec>(x, bias, residual, out, rows, cols,
+                                                       dropout, s, st);
+    return dropres_fwd_launch<T, 1>(x, bias, residual, out, rows, cols, dropout, s, st);
+}
+
+template <typename T>
+int dropres_bwd_dispatch(const void* grad, void* dx, void* dbias, void* ws, int64_t rows,
+                         int64_t cols, bool dropout, const DropoutState& s, hipStream_t st) {
+    const int want = dbias ? 1 : 0;
+    int rc;
+    if (vector_ok<T>(cols, {grad, dx}))
+        rc = dropres_bwd_launch<T, Elem<T>::kPerVec>(grad, dx, ws, rows, cols, dropout, want, s,
+                                                     st);
+    else
+        rc = dropres_bwd_launch<T, 1>(grad, dx, ws, rows, cols, dropout, want, s, st);
+    if (rc != SLAPO_OK || !dbias) return rc;
+    return finish_colsum<T>((const float*)ws, dbias, rows, cols, st);
+}
+
+inline bool dims_ok(int64_t rows, int64_t cols) {
+    return rows > 0 && cols > 0 && rows <= (int64_t)1 << 40 && cols <= (int64_t)1 << 30;
+}
+
+}  // namespace
+
+#define SLAPO_DISPATCH_DTYPE(dtype, CALL)   \
+    switch (dtype) {                        \
+        case SLAPO_F32: return CALL(float); \
+        case SLAPO_F16: return CALL(f16_t); \
+        case SLAPO_BF16: return CALL(bf16_t); \
+        default: return SLAPO_ERR_DTYPE;    \
+    }
+
+extern "C" size_t slapo_amd_colsum_workspace_bytes(int64_t rows, int64_t cols) {
+    if (rows <= 0 || cols <= 0) return 0;
+    const int64_t n_partials = (rows + kRowsPerBlock - 1) / kRowsPerBlock;
+    return (size_t)n_partials * (size_t)cols * sizeof(float);
+}
+
+extern "C" int slapo_amd_bias_gelu_fwd(const void* y, const void* bias, void* out, int64_t rows,
+                                       int64_t cols, int dtype, void* stream) {
+    if (!y || !bias || !out) return SLAPO_ERR_ARG;
+    if (!dims_ok(rows, cols)) return SLAPO_ERR_SHAPE;
+    hipStream_t st = (hipStream_t)stream;
+#define CALL(T) gelu_fwd_dispatch<T>(y, bias, out, rows, cols, st)
+    SLAPO_DISPATCH_DTYPE(dtype, CALL)
+#undef CALL
+}
+
+extern "C" int slapo_amd_bias_gelu_bwd(const void* grad, const void* y, const void* bias,
+                                       void* dx, void* dbias, void* workspace,
+                                       size_t workspace_bytes, int64_t rows, int64_t cols,
+                                       int dtype, void* stream) {
+    if (!grad || !y || !bias || !dx) return SLAPO_ERR_ARG;
+    if (!dims_ok(rows, cols)) return SLAPO_ERR_SHAPE;
+    if (dbias && (!workspace || workspace_bytes < slapo_amd_colsum_workspace_bytes(rows, cols)))
+        return SLAPO_ERR_WORKSPACE;
+    hipStream_t st = (hipStream_t)stream;
+#define CALL(T) gelu_bwd_dispatch<T>(grad, y, bias, dx, dbias, workspace, rows, cols, st)
+    SLAPO_DISPATCH_DTYPE(dtype, CALL)
+#undef CALL
+}
+
+extern "C" int slapo_amd_bias_dropout_residual_fwd(const void* x, const void* bias,
+                                                   const void* residual, void* out, int64_t rows,
+                                                   int64_t cols, int dtype, double p,
+                                                   uint64_t seed, uint64_t offset,
+                                                   const slapo_dropout_plan* plan, void* stream) {
+    if (!x || !bias || !out) return SLAPO_ERR_ARG;
+    if (!dims_ok(rows, cols)) return SLAPO_ERR_SHAPE;
+    if (!(p >= 0.0 && p <= 1.0)) return SLAPO_ERR_ARG;
+    const bool dropout = p > 0.0;
+    DropoutState s = {};
+    if (dropout) {
+        if (!plan_ok(plan, rows * cols)) return SLAPO_ERR_ARG;
+        s = make_dropout_state(*plan, p, seed, offset);
+    }
+    hipStream_t st = (hipStream_t)stream;
+#define CALL(T) dropres_fwd_dispatch<T>(x, bias, residual, out, rows, cols, dropout, s, st)
+    SLAPO_DISPATCH_DTYPE(dtype, CALL)
+#undef CALL
+}
+
+extern "C" int slapo_amd_bias_dropout_residual_bwd(const void* grad, void* dx, void* dbias,
+                                                   void* workspace, size_t workspace_bytes,
+                                                   int64_t rows, int64_t cols, int dtype,
+                                                   double p, uint64_t seed, uint64_t offset,
+                                                   const slapo_dropout_plan* plan, void* stream) {
+    if (!grad || (!dx && !dbias)) return SLAPO_ERR_ARG;
+    if (!dims_ok(rows, cols)) return SLAPO_ERR_SHAPE;
+    if (!(p >= 0.0 && p <= 1.0)) return SLAPO_ERR_ARG;
+    if (dbias && (!workspace || workspace_bytes < slapo_amd_colsum_workspace_bytes(rows, cols)))
+        return SLAPO_ERR_WORKSPACE;
+    const bool dropout = p > 0.0;
+    DropoutState s = {};
+    if (dropout) {
+        if (!plan_ok(plan, rows * cols)) return SLAPO_ERR_ARG;
+        s = make_dropout_state(*plan, p, seed, offset);
+    }
+    hipStream_t st = (hipStream_t)stream;
+#define CALL(T) dropres_bwd_dispatch<T>(grad, dx, dbias, workspace, rows, cols, dropout, s, st)
+    SLAPO_DISPATCH_DTYPE(dtype, CALL)
+#undef CALL
+}

@@ -1,0 +1,240 @@
+"""Tensor-level wrappers over the C ABI: argument checking, output/workspace allocation with
+torch's caching allocator, stream selection.  No arithmetic happens here."""
+from __future__ import annotations
+
+import ctypes
+import functools
+
+import torch
+
+from .. import _lib
+from .._lib import AttnParams, DropoutPlan
+
+
+def _require_device(*tensors):
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise RuntimeError(
+                "slapo_amd kernels run on a gfx950 device only; got a tensor on "
+                f"'{t.device}'.  There is no CPU implementation in this package."
+            )
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
+
+
+@functools.lru_cache(maxsize=4096)
+def _plan_cached(numel: int, elem_bytes: int, device_index: int):
+    plan = DropoutPlan()
+    rc = _lib.load().slapo_amd_dropout_plan(numel, elem_bytes, 256, device_index,
+                                            ctypes.byref(plan))
+    _lib.check(rc, "slapo_amd_dropout_plan")
+    return plan
+
+
+def dropout_plan(numel: int, elem_bytes: int, device) -> DropoutPlan:
+    """Launch plan torch.nn.functional.dropout would use for a fresh dense tensor."""
+    idx = torch.device(device).index
+    if idx is None:
+        idx = torch.cuda.current_device()
+    return _plan_cached(int(numel), int(elem_bytes), int(idx))
+
+
+def _rows_cols(x, bias):
+    cols = x.shape[-1]
+    if bias.ndim != 1 or bias.shape[0] != cols:
+        raise ValueError(f"bias must have shape [{cols}], got {tuple(bias.shape)}")
+    return x.numel() // cols, cols
+
+
+def _same_dtype(x, *others):
+    return [o if o is None or o.dtype == x.dtype else o.to(x.dtype) for o in others]
+
+
+def bias_gelu_fwd(y, bias):
+    _require_device(y, bias)
+    y = y.contiguous()
+    (bias,) = _same_dtype(y, bias.contiguous())
+    rows, cols = _rows_cols(y, bias)
+    out = torch.empty_like(y)
+    if y.numel() == 0:
+        return out
+    with torch.cuda.device(y.device):
+        rc = _lib.load().slapo_amd_bias_gelu_fwd(_ptr(y), _ptr(bias), _ptr(out), rows, cols,
+                                                 _lib.dtype_code(y.dtype), _stream())
+    _lib.check(rc, "slapo_amd_bias_gelu_fwd")
+    return out
+
+
+def _colsum_ws(rows, cols, device):
+    nbytes = _lib.load().slapo_amd_colsum_workspace_bytes(rows, cols)
+    return torch.empty(max(nbytes // 4, 1), dtype=torch.float32, device=device), nbytes
+
+
+def bias_gelu_bwd(grad, y, bias, need_dbias=True):
+    _require_device(grad, y, bias)
+    y = y.contiguous()
+    grad, bias = _same_dtype(y, grad.contiguous(), bias.contiguous())
+    rows, cols = _rows_cols(y, bias)
+    dx = torch.empty_like(y)
+    dbias = torch.empty_like(bias) if need_dbias else None
+    if y.numel() == 0:
+        return dx, (dbias.zero_() if dbias is not None else None)
+    with torch.cuda.device(y.device):
+        ws, nbytes = _colsum_ws(rows, cols, y.device) if need_dbias else (None, 0)
+        rc = _lib.load().slapo_amd_bias_gelu_bwd(_ptr(grad), _ptr(y), _ptr(bias), _ptr(dx),
+                                                 _ptr(dbias), _ptr(ws), nbytes, rows, cols,
+                                                 _lib.dtype_code(y.dtype), _stream())
+    _lib.check(rc, "slapo_amd_bias_gelu_bwd")
+    return dx, dbias
+
+
+def bias_dropout_residual_fwd(x, bias, residual, p, seed, offset, plan):
+    _require_device(x, bias, residual)
+    x = x.contiguous()
+    bias, residual = _same_dtype(x, bias.contiguous(),
+                                 residual.contiguous() if residual is not None else None)
+    if residual is not None and residual.shape != x.shape:
+        raise ValueError("residual must have the shape of x")
+    rows, cols = _rows_cols(x, bias)
+    out = torch.empty_like(x)
+    if x.numel() == 0:
+        return out
+    with torch.cuda.device(x.device):
+        rc = _lib.load().slapo_amd_bias_dropout_residual_fwd(
+            _ptr(x), _ptr(bias), _ptr(residual), _ptr(out), rows, cols,
+            _lib.dtype_code(x.dtype), float(p), seed, offset,
+            ctypes.byref(plan) if plan is not None else None, _stream())
+    _lib.check(rc, "slapo_amd_bias_dropout_residual_fwd")
+    return out
+
+
+def bias_dropout_residual_bwd(grad, bias_like, p, seed, offset, plan, need_dx=True,
+                              need_dbias=True):
+    _require_device(grad)
+    grad = grad.contiguous()
+    cols = grad.shape[-1]
+    rows = grad.numel() // cols
+    dx = torch.empty_like(grad) if need_dx else None
+    dbias = torch.empty(cols, dtype=grad.dtype, device=grad.device) if need_dbias else None
+    if grad.numel() == 0 or not (need_dx or need_dbias):
+        return dx, (dbias.zero_() if dbias is not None else None)
+    with torch.cuda.device(grad.device):
+        ws, nbytes = _colsum_ws(rows, cols, grad.device) if need_dbias else (None, 0)
+        rc = _lib.load().slapo_amd_bias_dropout_residual_bwd(
+            _ptr(grad), _ptr(dx), _ptr(dbias), _ptr(ws), nbytes, rows, cols,
+            _lib.dtype_code(grad.dtype), float(p), seed, offset,
+            ctypes.byref(plan) if plan is not None else None, _stream())
+    _lib.check(rc, "slapo_amd_bias_dropout_residual_bwd")
+    if dbias is not None and dbias.dtype != bias_like.dtype:
+        dbias = dbias.to(bias_like.dtype)
+    return dx, dbias
+
+
+def dropout_mask(numel, elem_bytes, p, seed, offset, device):
+    """Boolean keep-mask [numel] drawn on the device (debugging / test aid)."""
+    plan = dropout_plan(numel, elem_bytes, device)
+    mask = torch.empty(numel, dtype=torch.uint8, device=device)
+    with torch.cuda.device(device):
+        rc = _lib.load().slapo_amd_dropout_mask(_ptr(mask), ctypes.byref(plan), float(p), seed,
+                                                offset, _stream())
+    _lib.check(rc, "slapo_amd_dropout_mask")
+    return mask.bool()
+
+
+# ------------------------------------------------------------------------------------------
+# attention
+# ------------------------------------------------------------------------------------------
+def _bshd_strides(t):
+    if t.ndim != 4:
+        raise ValueError("attention operands must be [batch, seqlen, heads, head_dim]")
+    if t.shape[-1] > 1 and t.stride(-1) != 1:
+        raise ValueError("head_dim must be contiguous")
+    return (ctypes.c_int64 * 3)(t.stride(0), t.stride(1), t.stride(2))
+
+
+def _usable_layout(t):
+    """Strided [B,S,H,D] views are consumed as they are when rows stay 16-byte aligned."""
+    if t.stride(-1) != 1 and t.shape[-1] > 1:
+        return t.contiguous()
+    esz = t.element_size()
+    if (t.data_ptr() % 16) or any((s * esz) % 16 for s in t.stride()[:3]):
+        return t.contiguous()
+    return t
+
+
+def make_attn_params(q, k, v, o, bias, causal, window, scale, p, seed, offset, plan):
+    prm = AttnParams()
+    b, sq, h, d = q.shape
+    prm.dtype = _lib.dtype_code(q.dtype)
+    prm.batch, prm.heads, prm.seqlen_q, prm.seqlen_k, prm.head_dim = b, h, sq, k.shape[1], d
+    prm.causal = 1 if causal else 0
+    prm.window = int(window) if window else 0
+    prm.scale = float(scale)
+    prm.p_drop = float(p)
+    prm.seed = int(seed)
+    prm.offset = int(offset)
+    prm.q_strides = _bshd_strides(q)
+    prm.k_strides = _bshd_strides(k)
+    prm.v_strides = _bshd_strides(v)
+    prm.o_strides = _bshd_strides(o)
+    if bias is not None:
+        prm.bias_strides = (ctypes.c_int64 * 4)(*bias.stride())
+    if plan is not None:
+        prm.plan = plan
+    return prm
+
+
+def prepare_bias(attention_mask, b, h, sq, sk):
+    """Additive mask -> fp32 tensor viewed as [B,H,Sq,Sk] with stride 0 on broadcast dims."""
+    if attention_mask is None:
+        return None
+    m = attention_mask
+    if m.ndim != 4:
+        raise ValueError("attention_mask must be 4-D ([B,1,1,Sk] or [B,H,Sq,Sk])")
+    m = m.float() if m.dtype != torch.float32 else m
+    return m.expand(b, h, sq, sk)
+
+
+def attn_fwd(q, k, v, bias, causal, window, scale, p, seed, offset, plan):
+    _require_device(q, k, v, bias)
+    q, k, v = _usable_layout(q), _usable_layout(k), _usable_layout(v)
+    b, sq, h, d = q.shape
+    o = torch.empty((b, sq, h, d), dtype=q.dtype, device=q.device)
+    lse = torch.empty((b, h, sq), dtype=torch.float32, device=q.device)
+    prm = make_attn_params(q, k, v, o, bias, causal, window, scale, p, seed, offset, plan)
+    if o.numel():
+        with torch.cuda.device(q.device):
+            rc = _lib.load().slapo_amd_attn_fwd(ctypes.byref(prm), _ptr(q), _ptr(k), _ptr(v),
+                                                _ptr(bias), _ptr(o), _ptr(lse), _stream())
+        _lib.check(rc, "slapo_amd_attn_fwd")
+    return o, lse, (q, k, v)
+
+
+def attn_bwd(dout, q, k, v, bias, o, lse, causal, window, scale, p, seed, offset, plan):
+    _require_device(dout, q, k, v, o, lse, bias)
+    dout = dout if dout.stride() == o.stride() else dout.contiguous()
+    if dout.stride() != o.stride():
+        o = o.contiguous()
+    dq = torch.empty(q.shape, dtype=q.dtype, device=q.device)
+    dk = torch.empty(k.shape, dtype=k.dtype, device=k.device)
+    dv = torch.empty(v.shape, dtype=v.dtype, device=v.device)
+    prm = make_attn_params(q, k, v, o, bias, causal, window, scale, p, seed, offset, plan)
+    if dq.numel() and dk.numel():
+        lib = _lib.load()
+        nbytes = lib.slapo_amd_attn_bwd_workspace_bytes(ctypes.byref(prm))
+        with torch.cuda.device(q.device):
+            ws = torch.empty(max(nbytes // 4, 1), dtype=torch.float32, device=q.device)
+            rc = lib.slapo_amd_attn_bwd(
+                ctypes.byref(prm), _ptr(q), _ptr(k), _ptr(v), _ptr(bias), _ptr(o), _ptr(dout),
+                _ptr(lse), _ptr(dq), _ptr(dk), _ptr(dv), _bshd_strides(dq), _bshd_strides(dk),
+                _bshd_strides(dv), _ptr(ws), nbytes, _stream())
+        _lib.check(rc, "slapo_amd_attn_bwd")
+    else:
+        dq.zero_(), dk.zero_(), dv.zero_()
+    return dq, dk, dv

@@ -1,0 +1,118 @@
+"""Bias epilogues fused with the following activation / dropout, on hand-written HIP kernels.
+
+Same public names and call signatures as the reference's slapo/op/fused_bias.py
+(`BiasGeLUFunction` :13-46, `bias_new_gelu` :63-64, `bias_dropout` :67-74); each runs as ONE
+streaming kernel per direction instead of a TorchScript / functorch fusion.  Two modules,
+`HipBiasGeLU` and `HipBiasDropoutResidual`, package them with the positional signatures
+(`forward(x, bias)`, `forward(x, bias, residual)`) that `sch.replace(module, subgraph)` needs
+for the fusion patterns of tests/test_fusion.py:118-204.
+"""
+from __future__ import annotations
+
+import torch
+from torch import nn
+
+from ..random import draw_philox
+from . import _kernels as K
+
+
+class BiasGeLUFunction(torch.autograd.Function):
+    """gelu_tanh(inp + bias); backward is the closed form of fused_bias.py:26-34 and returns the
+    bias gradient already reduced to the bias shape."""
+
+    # pylint: disable=arguments-differ, abstract-method
+    @staticmethod
+    def forward(ctx, inp, bias):
+        ctx.save_for_backward(inp, bias)
+        return K.bias_gelu_fwd(inp, bias)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        inp, bias = ctx.saved_tensors
+        dx, dbias = K.bias_gelu_bwd(grad_output, inp, bias, need_dbias=ctx.needs_input_grad[1])
+        if dbias is not None and dbias.dtype != bias.dtype:
+            dbias = dbias.to(bias.dtype)
+        return (dx if ctx.needs_input_grad[0] else None), dbias
+
+
+def bias_gelu(inp: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
+    return BiasGeLUFunction.apply(inp, bias)
+
+
+def bias_new_gelu(inp: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
+    """HF `gelu_new` on inp + bias.  Its constant sqrt(2/pi) equals the 0.79788456 of
+    `BiasGeLUFunction` to 8 digits, so both names share one kernel."""
+    return BiasGeLUFunction.apply(inp, bias)
+
+
+class _BiasDropoutResidual(torch.autograd.Function):
+    # pylint: disable=arguments-differ, abstract-method
+    @staticmethod
+    def forward(ctx, x, bias, residual, p):
+        plan, seed, offset = None, 0, 0
+        if 0.0 < p:
+            plan = K.dropout_plan(x.numel(), x.element_size(), x.device)
+            if p < 1.0:
+                # The generator moves exactly as it would for F.dropout on this tensor.
+                seed, offset = draw_philox(plan.offset_increment, x.device)
+        ctx.p, ctx.seed, ctx.offset, ctx.plan = p, seed, offset, plan
+        ctx.bias_like = bias
+        ctx.has_residual = residual is not None
+        return K.bias_dropout_residual_fwd(x, bias, residual, p, seed, offset, plan)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        need_dx, need_dbias = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
+        dx = dbias = None
+        if need_dx or need_dbias:
+            if ctx.p == 0.0 and not need_dbias:
+                dx = grad_output
+            else:
+                dx, dbias = K.bias_dropout_residual_bwd(
+                    grad_output, ctx.bias_like, ctx.p, ctx.seed, ctx.offset, ctx.plan,
+                    need_dx=need_dx, need_dbias=need_dbias)
+        dres = grad_output if (ctx.has_residual and ctx.needs_input_grad[2]) else None
+        return dx, dbias, dres, None
+
+
+def bias_dropout(x: torch.Tensor, bias: torch.Tensor, p: float = 0.5, training: bool = True,
+                 inplace: bool = False) -> torch.Tensor:
+    """dropout(x + bias).  `inplace` is accepted for signature compatibility; the reference's
+    in-place target is the temporary x + bias, which this kernel never materialises."""
+    del inplace
+    _check_p(p)
+    return _BiasDropoutResidual.apply(x, bias, None, float(p) if training else 0.0)
+
+
+def bias_dropout_residual(x: torch.Tensor, bias: torch.Tensor, residual: torch.Tensor,
+                          p: float = 0.5, training: bool = True) -> torch.Tensor:
+    """dropout(x + bias) + residual, the pattern of tests/test_fusion.py:179-180."""
+    _check_p(p)
+    return _BiasDropoutResidual.apply(x, bias, residual, float(p) if training else 0.0)
+
+
+def _check_p(p):
+    if p < 0.0 or p > 1.0:
+        raise ValueError(f"dropout probability has to be between 0 and 1, but got {p}")
+
+
+class HipBiasGeLU(nn.Module):
+    """Replacement payload for a matched `gelu(x + bias)` subgraph."""
+
+    def forward(self, x, bias):
+        return BiasGeLUFunction.apply(x, bias)
+
+
+class HipBiasDropoutResidual(nn.Module):
+    """Replacement payload for a matched `dropout(x + bias) + residual` subgraph."""
+
+    def __init__(self, p: float = 0.5):
+        super().__init__()
+        _check_p(p)
+        self.p = p
+
+    def forward(self, x, bias, residual):
+        return bias_dropout_residual(x, bias, residual, self.p, self.training)
+
+    def extra_repr(self):
+        return f"p={self.p}"
