@@ -1,0 +1,73 @@
+"""Module-level parity on the GPU: FlashAttention / FlashAttentionOp as schedules install them,
+against an oracle composite built from the same weights (restates tests/test_op.py::test_attention,
+whose bar is atol = rtol = 5e-2 in fp16)."""
+import pytest
+import torch
+
+from oracle import attention as OA
+from slapo_amd import op
+from tests.conftest import assert_parity
+
+pytestmark = pytest.mark.gpu
+
+
+def _oracle_block(m, x, mask):
+    """QKV GEMM with the head-interleaved [H, 3, D] packing, oracle attention, out_proj."""
+    w = {n: p.detach().cpu().double() for n, p in m.named_parameters()}
+    b, s, _ = x.shape
+    h, d = m.num_attention_heads, m.attention_head_size
+    if m.fused_qkv:
+        packed = (x @ w["qkv.weight"].t() + w["qkv.bias"]).view(b, s, h, 3 * d)
+        q, k, v = packed.split(d, dim=-1)
+    else:
+        q, k, v = ((x @ w[f"{n}.weight"].t() + w[f"{n}.bias"]).view(b, s, h, d)
+                   for n in ("query", "key", "value"))
+    ctx = OA.xformers_ref(q, k, v, mask, m.output_proj, compute_dtype=torch.float64)
+    ctx = ctx.reshape(b, s, h * d)
+    if m.output_proj:
+        ctx = ctx @ w["out_proj.weight"].t() + w["out_proj.bias"]
+    return ctx
+
+
+@pytest.mark.parametrize("fused_qkv,output_proj", [(True, True), (False, True), (False, False)])
+def test_flash_attention_module_fwd_bwd(fused_qkv, output_proj):
+    torch.manual_seed(0)
+    b, s, hidden, heads = 2, 256, 512, 8
+    m = op.FlashAttention(hidden_size=hidden, num_attention_heads=heads, output_proj=output_proj,
+                          attn_pdrop=0.0, resid_pdrop=0.0, attn_op_name="hip_cdna4",
+                          fused_qkv=fused_qkv).half().cuda()
+    x = torch.randn(b, s, hidden, dtype=torch.float16, device="cuda", requires_grad=True)
+    mask = torch.randn(b, 1, 1, s, dtype=torch.float16, device="cuda", requires_grad=True)
+    out, present = m(x, mask, None)
+    assert present is None and out.shape == (b, s, hidden)
+    out.backward(torch.ones_like(out))
+    xr = x.detach().cpu().double().requires_grad_(True)
+    ref = _oracle_block(m, xr, mask.detach().cpu().double())
+    ref.backward(torch.ones_like(ref))
+    torch.testing.assert_close(out.detach().cpu().double(), ref.detach(), atol=5e-2, rtol=5e-2)
+    torch.testing.assert_close(x.grad.cpu().double(), xr.grad, atol=5e-2, rtol=5e-2)
+    assert mask.grad is None  # bias gradient is not produced (as in the reference)
+    out2, present = m(x, mask, None, use_cache=True)
+    assert present[0].shape == (b, s, heads, hidden // heads)
+
+
+def test_flash_attention_op_replacement_call():
+    """The tutorial's subgraph replacement calls the op with concrete_args attention_mask=None,
+    p=0.1 (docs/source/scripts/attention-single-gpu.py:279-282)."""
+    core = op.FlashAttentionOp("hip_cdna4", apply_causal_mask=False)
+    q, k, v = (torch.randn(2, 64, 4, 64, device="cuda", dtype=torch.bfloat16) for _ in range(3))
+    out = core(q, k, v, None, 0.0)
+    ref = OA.xformers_ref(q.cpu(), k.cpu(), v.cpu(), None, False, compute_dtype=torch.float64)
+    assert_parity(out, ref, torch.bfloat16, "op forward")
+    assert core(q, k, v, None, 0.1).shape == q.shape
+
+
+def test_window_kwarg_local_attention_module():
+    m = op.FlashAttention(128, 2, attn_op_name="hip_cdna4", fused_qkv=True, window=16).half().cuda()
+    x = torch.randn(1, 96, 128, dtype=torch.float16, device="cuda")
+    out, _ = m(x)
+    mg = op.FlashAttention(128, 2, attn_op_name="hip_cdna4", fused_qkv=True).half().cuda()
+    mg.load_state_dict(m.state_dict())
+    out_g, _ = mg(x)
+    # the first `window` positions see the same keys under both masks, later ones do not
+    assert torch.equal(out[:, :16], out_g[:, :16]) and not torch.equal(out[:, 16:], out_g[:, 16:])

@@ -1,0 +1,192 @@
+"""Host-side mirror of the reference's operator interface (CPU only): constructor signatures,
+attribute / child names, error behaviour, class-name contract, RNG tracker state machine.
+Assertions restate what the reference's callers rely on (slapo/model_schedule/gpt2.py:212-239,
+:452-520; slapo/tracer.py:626-635; tests/test_random.py:23-63)."""
+import inspect
+
+import pytest
+import torch
+from torch import nn
+
+import slapo_amd
+from slapo_amd import op
+from slapo_amd.random import CudaRNGStatesTracker
+
+
+def _params(fn):
+    return [(p.name, p.default) for p in inspect.signature(fn).parameters.values()
+            if p.name != "self"]
+
+
+def test_constructor_and_forward_signatures():
+    E = inspect.Parameter.empty
+    assert _params(op.FlashAttentionOp.__init__)[:3] == [
+        ("attn_op_name", E), ("apply_causal_mask", E), ("scale", None)]
+    assert _params(op.FlashAttentionOp.forward) == [
+        ("query_layer", E), ("key_layer", E), ("value_layer", E), ("attention_mask", E), ("p", E)]
+    assert _params(op.FlashAttention.__init__)[:8] == [
+        ("hidden_size", E), ("num_attention_heads", E), ("attn_pdrop", 0.0), ("resid_pdrop", 0.0),
+        ("attn_op_name", "auto"), ("bias", True), ("output_proj", True), ("fused_qkv", False)]
+    assert _params(op.FlashAttention.forward) == [
+        ("hidden_states", E), ("attention_mask", None), ("layer_past", None), ("head_mask", None),
+        ("encoder_hidden_states", None), ("encoder_attention_mask", None), ("use_cache", False),
+        ("output_attentions", False)]
+    assert _params(op.FusedMLP.__init__) == [
+        ("hidden_size", E), ("intermediate_size", E), ("orig_act", E), ("resid_pdrop", E),
+        ("use_torchscript", False)]
+    assert _params(op.LinearWithAct.__init__) == [
+        ("in_features", E), ("out_features", E), ("bias", True), ("act_fn", "gelu"),
+        ("device", None), ("dtype", None), ("sync_fn", None)]
+    assert _params(op.LinearWithDropout.__init__) == [
+        ("in_features", E), ("out_features", E), ("bias", True), ("p", 0.5), ("inplace", False),
+        ("device", None), ("dtype", None), ("sync_fn", None), ("use_torchscript", False)]
+    assert _params(op.bias_dropout) == [
+        ("x", E), ("bias", E), ("p", 0.5), ("training", True), ("inplace", False)]
+
+
+def test_attention_module_children_and_attributes():
+    # kwargs exactly as the GPT-2 schedule passes them (model_schedule/gpt2.py:212-220)
+    m = op.FlashAttention(hidden_size=64, num_attention_heads=4, output_proj=True, attn_pdrop=0.1,
+                          resid_pdrop=0.1, attn_op_name="hip_cdna4", fused_qkv=True)
+    assert set(dict(m.named_children())) == {"qkv", "out_proj", "resid_dropout", "attn_op"}
+    assert m.qkv.out_features == 192 and m.attn_op.apply_causal_mask is True
+    assert m.bias_layout == m.attn_op.bias_layout == "b11k"
+    assert m.attn_op.pkg == "hip" and callable(m.attn_op.attn_fn)
+    # BERT style (model_schedule/bert.py:165-174): no projection -> bidirectional, separate q/k/v
+    e = op.FlashAttention(64, 4, output_proj=False, fused_qkv=False)
+    assert set(dict(e.named_children())) == {"query", "key", "value", "attn_op"}
+    assert e.attn_op.apply_causal_mask is False
+    mlp = op.FusedMLP(16, 64, "gelu_new", 0.1)
+    assert set(dict(mlp.named_children())) == {"fc_in", "fc_out"}
+    assert mlp.fc_in.act_fn == "gelu" and mlp.fc_out.p == 0.1
+    assert mlp.fc_in.sync_fn is None and mlp.fc_out.sync_fn is None
+    mlp.fc_out.sync_fn = lambda x: x  # schedules assign it after construction
+    assert "sync_fn=<lambda>" in repr(mlp.fc_out)
+
+
+def test_class_name_contract_for_leaf_matching():
+    # the reference's tracer matches substrings of type(m).__name__
+    assert "FlashAttentionOp" in type(op.FlashAttentionOp("hip_cdna4", True)).__name__
+    assert "LinearWithAct" in type(op.LinearWithAct(4, 4)).__name__
+    assert "LinearWithDropout" in type(op.LinearWithDropout(4, 4)).__name__
+    assert op.LinearWithSyncFunc(4, 4).traceable is False
+
+
+def test_error_behaviour():
+    with pytest.raises(ValueError):
+        op.FlashAttention(30, 4)
+    with pytest.raises(ValueError):
+        op.FlashAttentionOp("no_such_kernel", True)
+    with pytest.raises(ValueError):
+        op.FlashAttentionOp("native_xformers", True)
+    with pytest.raises(ValueError):
+        op.LinearWithAct(4, 4, bias=False)
+    with pytest.raises(ValueError):
+        op.LinearWithDropout(4, 4, bias=False)
+    with pytest.raises(NotImplementedError):
+        op.LinearWithAct(4, 4, act_fn="relu")
+    m = op.FlashAttention(16, 2, attn_op_name="hip_cdna4")
+    x = torch.zeros(1, 4, 16)
+    with pytest.raises(NotImplementedError):
+        m(x, encoder_hidden_states=x)
+    with pytest.raises(NotImplementedError):
+        m(x, output_attentions=True)
+    with pytest.raises(NotImplementedError):
+        m(x, head_mask=torch.ones(2))
+
+
+def test_third_party_names_are_aliases():
+    # schedules fall back to "cutlass" when a constructor raises (gpt2.py:229-239)
+    for name in ("cutlass", "flash", "triton", "cuda", "small_k", "auto"):
+        assert op.FlashAttentionOp(name, True).pkg == "hip"
+
+
+def test_no_cpu_fallback():
+    """CPU tensors are refused loudly: the package has no eager substitute for its kernels."""
+    with pytest.raises(RuntimeError, match="gfx950"):
+        op.bias_gelu(torch.zeros(4, 8), torch.zeros(8))
+    with pytest.raises(RuntimeError, match="gfx950"):
+        op.bias_dropout(torch.zeros(4, 8), torch.zeros(8), 0.0, False)
+    with pytest.raises(RuntimeError, match="gfx950"):
+        op.hip_attention(*(torch.zeros(1, 8, 1, 8, dtype=torch.float16) for _ in range(3)))
+    mlp = op.FusedMLP(8, 32, "gelu", 0.0)
+    with pytest.raises(RuntimeError, match="gfx950"):
+        mlp(torch.zeros(2, 8))
+
+
+def test_meta_device_construction():
+    # schedules build the modules under init_empty_weights (gpt2.py:268-272)
+    with torch.device("meta"):
+        m = op.FlashAttention(64, 4, attn_op_name="hip_cdna4", fused_qkv=True)
+        f = op.FusedMLP(64, 256, "gelu", 0.1)
+    assert all(p.is_meta for p in list(m.parameters()) + list(f.parameters()))
+
+
+def test_separate_bias_linear_and_fused_qkv_on_cpu():
+    lin = op.LinearWithSeparateBias(6, 5)
+    x = torch.randn(3, 6)
+    torch.testing.assert_close(lin(x), nn.functional.linear(x, lin.weight, lin.bias))
+    sync = op.LinearWithSyncFunc(6, 5, sync_fn=lambda t: t * 2)
+    torch.testing.assert_close(sync(x), nn.functional.linear(x, sync.weight) * 2 + sync.bias)
+    qkv = op.FusedQKV(8, 2, 1)
+    q, k, v = qkv(torch.randn(2, 3, 8))
+    assert q.shape == k.shape == v.shape == (2, 3, 2, 4)
+
+
+class _FakeBackend:
+    """Stands in for the device generator: state = (seed, offset)."""
+
+    def __init__(self):
+        self.state = (0, 0)
+
+    def get_state(self):
+        return self.state
+
+    def set_state(self, s):
+        self.state = s
+
+    def manual_seed(self, seed):
+        self.state = (seed, 0)
+
+    def draw(self, n=4):
+        s = self.state
+        self.state = (s[0], s[1] + n)
+        return s
+
+
+def test_rng_tracker_state_machine():
+    be = _FakeBackend()
+    tr = CudaRNGStatesTracker(be)
+    be.manual_seed(2013)
+    be.draw()
+    tr.add("model-parallel-rng", 2013 + 2718)
+    assert be.state == (2013, 4)  # add() leaves the outer stream untouched
+    with pytest.raises(Exception, match="seed 4731 already exists"):
+        tr.add("other", 4731)
+    with pytest.raises(Exception, match="already exists"):
+        tr.add("model-parallel-rng", 1)
+    with pytest.raises(RuntimeError, match="is not added"):
+        with tr.fork("missing"):
+            pass
+    with tr.fork():
+        assert be.draw() == (4731, 0)
+    with tr.fork():
+        assert be.draw() == (4731, 4)  # the named stream continues where it stopped
+    assert be.state == (2013, 4)       # and the outer one never moved
+    try:
+        with tr.fork():
+            be.draw()
+            raise KeyError
+    except KeyError:
+        pass
+    assert be.state == (2013, 4) and tr.get_states()["model-parallel-rng"] == (4731, 12)
+    tr.reset()
+    assert not tr.get_states()
+
+
+def test_set_random_seed_arithmetic():
+    assert slapo_amd.set_random_seed(2013) == 2013
+    assert slapo_amd.set_random_seed(2013, dp_rank=3, pp_rank=2) == 2013 + 200 + 30
+    a = torch.rand(3)
+    slapo_amd.set_random_seed(2013, dp_rank=3, pp_rank=2)
+    torch.testing.assert_close(torch.rand(3), a)
