@@ -1,0 +1,267 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused-op hot path on ONE MI355X.
+
+A "step" is one forward + backward pass of the attention op over one batch of the workload
+"GPT-2-medium-shaped causal attention": fp16, batch 8, seq 1024, 16 heads x 64, causal, dropout 0,
+Q/K/V/dO ~ N(0,1) from seed 2013 (synthetic).  All tensors are resident in HBM before the timed
+region; the kernels are called through the C ABI (libslapo_amd.so) with preallocated outputs.
+
+value     attention fwd+bwd TFLOP/s = 14 * D * N / time per step, N = attended (query, key) pairs
+roofline  the backward MFMA kernel (the dominant kernel): its algorithmic FLOPs (10 * D * N) over
+          its own average launch duration, taken with HIP events placed around the MAIN stage of
+          the backward on the launching stream, against the dense fp16 MFMA peak
+epilogue  GB/s of the two FusedMLP epilogues (bf16, tokens 8192, 1024 -> 4096 -> 1024) against the
+          HBM peak, on a rotating working set larger than the caches
+cpu_baseline  the oracle's native-PyTorch restatement (fp32 CPU, autograd backward) timed on the
+          host cores on a bounded sample of the same workload
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 / bf16
+HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
+
+WORKLOAD = dict(name="gpt2-medium causal attention fwd+bwd", dtype="fp16", batch=8, seq=1024,
+                heads=16, head_dim=64, causal=True, p=0.0, seed=2013)
+
+
+def _pairs(seq, causal):
+    return seq * (seq + 1) // 2 if causal else seq * seq
+
+
+def _make_inputs(cfg, device):
+    g = torch.Generator().manual_seed(cfg["seed"])
+    shape = (cfg["batch"], cfg["seq"], cfg["heads"], cfg["head_dim"])
+    return [torch.randn(shape, generator=g).to(torch.float16).to(device) for _ in range(4)]
+
+
+class AttentionStep:
+    """Forward + backward of the attention op through the C ABI on preallocated buffers."""
+
+    def __init__(self, cfg, device):
+        from slapo_amd import _lib
+        from slapo_amd.op import _kernels as K
+
+        self.lib = _lib.load()
+        self._lib_mod = _lib
+        self.q, self.k, self.v, self.do = _make_inputs(cfg, device)
+        q = self.q
+        self.o = torch.empty_like(q)
+        self.lse = torch.empty(cfg["batch"], cfg["heads"], cfg["seq"], dtype=torch.float32,
+                               device=device)
+        self.dq, self.dk, self.dv = (torch.empty_like(q) for _ in range(3))
+        self.prm = K.make_attn_params(self.q, self.k, self.v, self.o, None, cfg["causal"], 0,
+                                      cfg["head_dim"] ** -0.5, 0.0, 0, 0, None)
+        nbytes = self.lib.slapo_amd_attn_bwd_workspace_bytes(ctypes.byref(self.prm))
+        self.ws = torch.empty(nbytes // 4, dtype=torch.float32, device=device)
+        self.ws_bytes = nbytes
+        self.strides = [K._bshd_strides(t) for t in (self.dq, self.dk, self.dv)]
+        self.stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        P = lambda t: ctypes.c_void_p(t.data_ptr())
+        self.fwd_args = (ctypes.byref(self.prm), P(self.q), P(self.k), P(self.v), None, P(self.o),
+                         P(self.lse), self.stream)
+        self.bwd_args = (ctypes.byref(self.prm), P(self.q), P(self.k), P(self.v), None, P(self.o),
+                         P(self.do), P(self.lse), P(self.dq), P(self.dk), P(self.dv),
+                         *self.strides, P(self.ws), self.ws_bytes)
+
+    def forward(self):
+        rc = self.lib.slapo_amd_attn_fwd(*self.fwd_args)
+        if rc:
+            raise RuntimeError(f"slapo_amd_attn_fwd failed with status {rc}")
+
+    def backward(self, stages=7):
+        rc = self.lib.slapo_amd_attn_bwd_stages(*self.bwd_args, stages, self.stream)
+        if rc:
+            raise RuntimeError(f"slapo_amd_attn_bwd_stages failed with status {rc}")
+
+    def step(self, ev=None):
+        self.forward()
+        self.backward(self._lib_mod.BWD_PREPARE)
+        if ev is not None:
+            ev[0].record()
+        self.backward(self._lib_mod.BWD_MAIN)
+        if ev is not None:
+            ev[1].record()
+        self.backward(self._lib_mod.BWD_FINISH)
+
+
+def bench_epilogues(device, iters=40):
+    """GB/s of bias-GeLU fwd and bias-dropout-residual fwd on rotating buffers (> 1 GB)."""
+    from slapo_amd import _lib
+    from slapo_amd.op import _kernels as K
+
+    lib = _lib.load()
+    T, I, Hd = 8192, 4096, 1024
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    bf = torch.bfloat16
+    out = {}
+
+    def timed(fn, n_rot):
+        for i in range(n_rot):
+            fn(i)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(iters):
+            fn(i % n_rot)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / iters * 1e-3  # seconds per launch
+
+    n_rot = 8
+    ys = [torch.randn(T, I, device=device, dtype=bf) for _ in range(n_rot)]
+    outs = [torch.empty(T, I, device=device, dtype=bf) for _ in range(n_rot)]
+    b = torch.randn(I, device=device, dtype=bf)
+
+    def gelu(i):
+        rc = lib.slapo_amd_bias_gelu_fwd(P(ys[i]), P(b), P(outs[i]), T, I, _lib.SLAPO_BF16, st)
+        assert rc == 0
+
+    sec = timed(gelu, n_rot)
+    nbytes = 2 * T * I * 2 + I * 2
+    out["bias_gelu_fwd"] = {"bytes": nbytes, "us": sec * 1e6, "GBps": nbytes / sec / 1e9,
+                            "frac_of_hbm_peak": nbytes / sec / 1e9 / HBM_PEAK_GBS}
+
+    gos = outs
+
+    def gelu_bwd(i):
+        rc = lib.slapo_amd_bias_gelu_bwd(P(gos[i]), P(ys[i]), P(b), P(outs[(i + 1) % n_rot]),
+                                         P(db), P(ws), ws_bytes, T, I, _lib.SLAPO_BF16, st)
+        assert rc == 0
+
+    ws_bytes = lib.slapo_amd_colsum_workspace_bytes(T, I)
+    ws = torch.empty(ws_bytes // 4, dtype=torch.float32, device=device)
+    db = torch.empty(I, device=device, dtype=bf)
+    sec = timed(gelu_bwd, n_rot)
+    nbytes = 3 * T * I * 2 + 2 * I * 2
+    out["bias_gelu_bwd"] = {"bytes": nbytes, "us": sec * 1e6, "GBps": nbytes / sec / 1e9,
+                            "frac_of_hbm_peak": nbytes / sec / 1e9 / HBM_PEAK_GBS}
+    del ys, outs, gos
+
+    n_rot = 24
+    xs = [torch.randn(T, Hd, device=device, dtype=bf) for _ in range(n_rot)]
+    rs = [torch.randn(T, Hd, device=device, dtype=bf) for _ in range(n_rot)]
+    os_ = [torch.empty(T, Hd, device=device, dtype=bf) for _ in range(n_rot)]
+    b1 = torch.randn(Hd, device=device, dtype=bf)
+    plan = K.dropout_plan(T * Hd, 2, device)
+
+    def dropres(i):
+        rc = lib.slapo_amd_bias_dropout_residual_fwd(P(xs[i]), P(b1), P(rs[i]), P(os_[i]), T, Hd,
+                                                     _lib.SLAPO_BF16, 0.1, 2013, 0,
+                                                     ctypes.byref(plan), st)
+        assert rc == 0
+
+    sec = timed(dropres, n_rot)
+    nbytes = 3 * T * Hd * 2 + Hd * 2
+    out["bias_dropout_residual_fwd"] = {"bytes": nbytes, "us": sec * 1e6,
+                                        "GBps": nbytes / sec / 1e9,
+                                        "frac_of_hbm_peak": nbytes / sec / 1e9 / HBM_PEAK_GBS}
+    return out
+
+
+def cpu_baseline(cfg, budget_batches=8):
+    """The oracle's native path (fp32 CPU, autograd) on `budget_batches` of the 8 batches."""
+    from oracle import attention as OA
+
+    threads = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(threads)
+    g = torch.Generator().manual_seed(cfg["seed"])
+    shape = (budget_batches, cfg["seq"], cfg["heads"], cfg["head_dim"])
+    q, k, v, do = (torch.randn(shape, generator=g).to(torch.float16) for _ in range(4))
+
+    def run():
+        t0 = time.perf_counter()
+        OA.attention_fwd_bwd(q, k, v, do, None, cfg["causal"], compute_dtype=torch.float32)
+        return time.perf_counter() - t0
+
+    run()  # warm-up
+    times = sorted(run() for _ in range(3))
+    sec = times[1]
+    flops = 14 * cfg["head_dim"] * _pairs(cfg["seq"], cfg["causal"]) * budget_batches * cfg["heads"]
+    return {"value": flops / sec / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+            "sample": f"{budget_batches} of {cfg['batch']} batches of the same workload "
+                      f"(fp32 math on fp16 inputs, median of 3, {sec:.2f} s per pass)"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-epilogues", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU's throughput; --gpus above 1 is not supported "
+                 "(no collectives are part of this hot path)")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs an MI355X (no GPU visible)")
+
+    cfg = WORKLOAD
+    device = torch.device("cuda", 0)
+    torch.cuda.set_device(device)
+    step = AttentionStep(cfg, device)
+
+    for _ in range(args.warmup):
+        step.step()
+    torch.cuda.synchronize()
+    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+              for _ in range(args.steps)]
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step.step(events[i])
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+
+    n_pairs = _pairs(cfg["seq"], cfg["causal"]) * cfg["batch"] * cfg["heads"]
+    d = cfg["head_dim"]
+    ms_per_step = elapsed / args.steps * 1e3
+    value = 14 * d * n_pairs / (elapsed / args.steps) / 1e12
+    kern_ms = sum(a.elapsed_time(b) for a, b in events) / args.steps
+    bwd_flops = 10 * d * n_pairs
+    achieved = bwd_flops / (kern_ms * 1e-3) / 1e12
+
+    result = {
+        "metric": "attention fwd+bwd TFLOP/s + epilogue GB/s, % of MI355X roofline, 1 GPU",
+        "value": value,
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": cfg["name"], "batch": cfg["batch"], "seq_len": cfg["seq"],
+                   "heads": cfg["heads"], "head_dim": cfg["head_dim"], "causal": cfg["causal"],
+                   "dropout_p": cfg["p"], "flops_per_step": 14 * d * n_pairs},
+        "frac_of_mfma_peak": value / MFMA_PEAK_TFLOPS,
+        "roofline": {"bound": "mfma", "kernel": "attn_bwd_kernel<f16, 64>", "achieved": achieved,
+                     "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / MFMA_PEAK_TFLOPS, "traffic": None,
+                     "flops_per_launch": bwd_flops, "avg_launch_ms": kern_ms},
+    }
+    if not args.no_epilogues:
+        result["epilogue"] = bench_epilogues(device)
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(cfg)
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

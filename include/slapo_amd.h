@@ -175,6 +175,24 @@ int slapo_amd_attn_bwd(const slapo_attn_params* prm, const void* q, const void* 
                        const int64_t dk_strides[3], const int64_t dv_strides[3], void* workspace,
                        size_t workspace_bytes, void* stream);
 
+/* The backward runs as three stages on `stream`: PREPARE (delta = rowsum(dO * O), clear the fp32
+ * dQ accumulator), MAIN (the dK / dV / dQ-accumulate kernel) and FINISH (dQ accumulator -> dq in
+ * the tensor dtype).  slapo_amd_attn_bwd runs all three; this entry point runs the stages named in
+ * `stages` (a bit-or of the constants below) so that a caller can place its own events around one
+ * of them or overlap PREPARE with other work.  Arguments are those of slapo_amd_attn_bwd and must
+ * be the same across the calls of one backward pass.  For SLAPO_F32 the MAIN stage writes dq
+ * directly and FINISH is a no-op. */
+#define SLAPO_BWD_PREPARE 1
+#define SLAPO_BWD_MAIN 2
+#define SLAPO_BWD_FINISH 4
+#define SLAPO_BWD_ALL 7
+int slapo_amd_attn_bwd_stages(const slapo_attn_params* prm, const void* q, const void* k,
+                              const void* v, const float* bias, const void* o, const void* dout,
+                              const float* lse, void* dq, void* dk, void* dv,
+                              const int64_t dq_strides[3], const int64_t dk_strides[3],
+                              const int64_t dv_strides[3], void* workspace,
+                              size_t workspace_bytes, int stages, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -109,7 +109,15 @@ PROTOTYPES = {
          ctypes.POINTER(c_i64), ctypes.POINTER(c_i64), ctypes.POINTER(c_i64), c_vp,
          ctypes.c_size_t, c_vp],
     ),
+    "slapo_amd_attn_bwd_stages": (
+        ctypes.c_int,
+        [ctypes.POINTER(AttnParams), c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp,
+         ctypes.POINTER(c_i64), ctypes.POINTER(c_i64), ctypes.POINTER(c_i64), c_vp,
+         ctypes.c_size_t, ctypes.c_int, c_vp],
+    ),
 }
+
+BWD_PREPARE, BWD_MAIN, BWD_FINISH, BWD_ALL = 1, 2, 4, 7
 
 _lib = None
 _lock = threading.Lock()

@@ -178,18 +178,20 @@ extern "C" size_t slapo_amd_attn_bwd_workspace_bytes(const slapo_attn_params* pr
     return bytes;
 }
 
-extern "C" int slapo_amd_attn_bwd(const slapo_attn_params* prm, const void* q, const void* k,
-                                  const void* v, const float* bias, const void* o,
-                                  const void* dout, const float* lse, void* dq, void* dk,
-                                  void* dv, const int64_t dq_strides[3],
-                                  const int64_t dk_strides[3], const int64_t dv_strides[3],
-                                  void* workspace, size_t workspace_bytes, void* stream) {
+extern "C" int slapo_amd_attn_bwd_stages(const slapo_attn_params* prm, const void* q,
+                                         const void* k, const void* v, const float* bias,
+                                         const void* o, const void* dout, const float* lse,
+                                         void* dq, void* dk, void* dv,
+                                         const int64_t dq_strides[3], const int64_t dk_strides[3],
+                                         const int64_t dv_strides[3], void* workspace,
+                                         size_t workspace_bytes, int stages, void* stream) {
     AttnArgs a = {};
     int rc = fill_args(prm, &a, true);
     if (rc != SLAPO_OK) return rc;
     if (!q || !k || !v || !o || !dout || !lse || !dq || !dk || !dv || !dq_strides ||
         !dk_strides || !dv_strides)
         return SLAPO_ERR_ARG;
+    if (stages <= 0 || stages > SLAPO_BWD_ALL) return SLAPO_ERR_ARG;
     if (!workspace || workspace_bytes < slapo_amd_attn_bwd_workspace_bytes(prm) ||
         !aligned16(workspace))
         return SLAPO_ERR_WORKSPACE;
@@ -211,19 +213,24 @@ extern "C" int slapo_amd_attn_bwd(const slapo_attn_params* prm, const void* q, c
     a.delta = is_f32 ? dq_acc : dq_acc + rows * a.d;
 
     if (is_f32) {
-        const bool vec_ok = a.d % 4 == 0 && aligned16(o) && aligned16(dout) &&
-                            strides_ok(prm->o_strides, 4);
-        if (vec_ok) {
-            const unsigned blocks = (unsigned)((rows * 8 + 255) / 256);
-            hipLaunchKernelGGL((attn_delta_kernel<float>), dim3(blocks), dim3(256), 0, st, a);
-        } else {
-            const unsigned blocks = (unsigned)((rows + 255) / 256);
-            hipLaunchKernelGGL(attn_delta_scalar_kernel, dim3(blocks), dim3(256), 0, st, a);
+        if (stages & SLAPO_BWD_PREPARE) {
+            const bool vec_ok = a.d % 4 == 0 && aligned16(o) && aligned16(dout) &&
+                                strides_ok(prm->o_strides, 4);
+            if (vec_ok) {
+                const unsigned blocks = (unsigned)((rows * 8 + 255) / 256);
+                hipLaunchKernelGGL((attn_delta_kernel<float>), dim3(blocks), dim3(256), 0, st, a);
+            } else {
+                const unsigned blocks = (unsigned)((rows + 255) / 256);
+                hipLaunchKernelGGL(attn_delta_scalar_kernel, dim3(blocks), dim3(256), 0, st, a);
+            }
+            rc = check_launch();
+            if (rc != SLAPO_OK) return rc;
         }
-        rc = check_launch();
-        if (rc != SLAPO_OK) return rc;
-        a.dq = dq;
-        return attn_bwd_f32(a, st);
+        if (stages & SLAPO_BWD_MAIN) {
+            a.dq = dq;
+            rc = attn_bwd_f32(a, st);
+        }
+        return rc;
     }
 
     if (!half_ptrs_ok({q, k, v, o, dout, dq, dk, dv})) return SLAPO_ERR_ALIGN;
@@ -231,26 +238,42 @@ extern "C" int slapo_amd_attn_bwd(const slapo_attn_params* prm, const void* q, c
         return SLAPO_ERR_ALIGN;
 
     const unsigned row_blocks = (unsigned)((rows * 8 + 255) / 256);
-    if (prm->dtype == SLAPO_F16)
-        hipLaunchKernelGGL((attn_delta_kernel<f16_t>), dim3(row_blocks), dim3(256), 0, st, a);
-    else
-        hipLaunchKernelGGL((attn_delta_kernel<bf16_t>), dim3(row_blocks), dim3(256), 0, st, a);
-    const int64_t n4 = rows * a.d / 4;  // head_dim % 8 == 0
-    hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, st,
-                       reinterpret_cast<f32x4_t*>(dq_acc), n4);
-    rc = check_launch();
-    if (rc != SLAPO_OK) return rc;
+    if (stages & SLAPO_BWD_PREPARE) {
+        if (prm->dtype == SLAPO_F16)
+            hipLaunchKernelGGL((attn_delta_kernel<f16_t>), dim3(row_blocks), dim3(256), 0, st, a);
+        else
+            hipLaunchKernelGGL((attn_delta_kernel<bf16_t>), dim3(row_blocks), dim3(256), 0, st, a);
+        const int64_t n4 = rows * a.d / 4;  // head_dim % 8 == 0
+        hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, st,
+                           reinterpret_cast<f32x4_t*>(dq_acc), n4);
+        rc = check_launch();
+        if (rc != SLAPO_OK) return rc;
+    }
+    if (stages & SLAPO_BWD_MAIN) {
+        a.dq = dq_acc;
+        rc = attn_bwd_mfma(a, prm->dtype, st);
+        if (rc != SLAPO_OK) return rc;
+    }
+    if (stages & SLAPO_BWD_FINISH) {
+        a.dq = dq;
+        if (prm->dtype == SLAPO_F16)
+            hipLaunchKernelGGL((dq_convert_kernel<f16_t>), dim3(row_blocks), dim3(256), 0, st, a,
+                               dq_acc);
+        else
+            hipLaunchKernelGGL((dq_convert_kernel<bf16_t>), dim3(row_blocks), dim3(256), 0, st, a,
+                               dq_acc);
+        rc = check_launch();
+    }
+    return rc;
+}
 
-    a.dq = dq_acc;
-    rc = attn_bwd_mfma(a, prm->dtype, st);
-    if (rc != SLAPO_OK) return rc;
-
-    a.dq = dq;
-    if (prm->dtype == SLAPO_F16)
-        hipLaunchKernelGGL((dq_convert_kernel<f16_t>), dim3(row_blocks), dim3(256), 0, st, a,
-                           dq_acc);
-    else
-        hipLaunchKernelGGL((dq_convert_kernel<bf16_t>), dim3(row_blocks), dim3(256), 0, st, a,
-                           dq_acc);
-    return check_launch();
+extern "C" int slapo_amd_attn_bwd(const slapo_attn_params* prm, const void* q, const void* k,
+                                  const void* v, const float* bias, const void* o,
+                                  const void* dout, const float* lse, void* dq, void* dk,
+                                  void* dv, const int64_t dq_strides[3],
+                                  const int64_t dk_strides[3], const int64_t dv_strides[3],
+                                  void* workspace, size_t workspace_bytes, void* stream) {
+    return slapo_amd_attn_bwd_stages(prm, q, k, v, bias, o, dout, lse, dq, dk, dv, dq_strides,
+                                     dk_strides, dv_strides, workspace, workspace_bytes,
+                                     SLAPO_BWD_ALL, stream);
 }
