@@ -34,6 +34,17 @@ HIPCC_FLAGS = [
 ]
 
 
+# The MFMA attention kernels never compute with NaNs on their defined paths (masked scores are
+# -inf, guarded before every subtraction); telling the compiler so removes the canonicalising
+# v_max x,x it would otherwise put in front of every max of an MFMA result.
+PER_FILE_FLAGS = {
+    "attn_fwd_f16.hip": ["-fno-honor-nans"],
+    "attn_fwd_bf16.hip": ["-fno-honor-nans"],
+    "attn_bwd_f16.hip": ["-fno-honor-nans"],
+    "attn_bwd_bf16.hip": ["-fno-honor-nans"],
+}
+
+
 def _hipcc() -> str:
     exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     if not os.path.exists(exe):
@@ -49,7 +60,8 @@ def sources() -> list[str]:
 
 def _compile_one(src: str, extra: list[str]) -> str:
     obj = os.path.join(OBJ_DIR, os.path.basename(src)[:-4] + ".o")
-    cmd = [_hipcc(), *HIPCC_FLAGS, *extra, "-c", src, "-o", obj]
+    per_file = PER_FILE_FLAGS.get(os.path.basename(src), [])
+    cmd = [_hipcc(), *HIPCC_FLAGS, *per_file, *extra, "-c", src, "-o", obj]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         raise RuntimeError(f"hipcc failed for {src}:\n{proc.stdout}\n{proc.stderr}")

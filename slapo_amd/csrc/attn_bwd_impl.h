@@ -23,13 +23,16 @@
 //                                    tile per workgroup and query tile instead of one per
 //                                    wavefront.
 // One barrier per query tile.  Reference semantics: autograd of slapo/op/attention.py:163-181.
+#pragma once
+#include <cstdio>
 #include <hip/amd_detail/amd_hip_unsafe_atomics.h>
+
+#include <type_traits>
 
 #include "attn_common.h"
 
-using namespace slapo;
-
-namespace {
+namespace slapo {
+namespace bwd {
 
 constexpr int kBwdWaves = 4;
 constexpr int kBwdThreads = kBwdWaves * 64;
@@ -52,7 +55,7 @@ struct BwdSmem {
     static constexpr size_t kBytes = kLoopBytes > kStageBytes ? kLoopBytes : kStageBytes;
 };
 
-template <typename T, int DPAD>
+template <typename T, int DPAD, bool kBias, bool kDropout>
 __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_kernel(
     const AttnArgs a) {
     typedef typename Mma<T>::frag frag_t;
@@ -82,6 +85,15 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
     const int wave = threadIdx.x >> 6;
     const int g = lane >> 5;
     const int c_loc = lane & 31;
+#ifdef EXP_TIMING
+    unsigned long long* tbuf = reinterpret_cast<unsigned long long*>(a.o) + 512;
+    int tcount = 0;
+    const bool trec = (blockIdx.x == EXP_TIMING) && threadIdx.x == 0;
+#define TSTAMP() do { if (trec) tbuf[tcount++] = __builtin_readcyclecounter(); } while (0)
+    TSTAMP();
+#else
+#define TSTAMP() do {} while (0)
+#endif
     const int kw0 = k0 + wave * 32;
     const int key = kw0 + c_loc;  // this lane's key column
 
@@ -111,6 +123,7 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
     {
         TileStage<T, DPAD, kBwdBN, kBwdThreads> kst;
         kst.load(k_base, a.ks[1], k0, a.sk, a.d);
+        kst.fix(k0, a.sk, a.d);
         kst.store(kstage);
         __syncthreads();
         const int beta = lane >> 4;
@@ -144,14 +157,23 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
     const int t_hi = (i_hi + kBwdBM - 1) / kBwdBM;
 
     // Per-lane bias when it does not depend on the query (the compact [B,1,1,Sk] layout).
-    const bool bias_per_key = a.has_bias && a.bs[2] == 0;
+    const bool bias_per_key = kBias && a.bs[2] == 0;
     float bias_k = 0.f;
-    if (bias_per_key && key < a.sk)
-        bias_k = a.bias[b * a.bs[0] + h * a.bs[1] + (int64_t)key * a.bs[3]] * kLog2e;
+    if constexpr (kBias) {
+        if (bias_per_key && key < a.sk)
+            bias_k = a.bias[b * a.bs[0] + h * a.bs[1] + (int64_t)key * a.bs[3]] * kLog2e;
+    }
+    const float c_log2 = a.scale_log2;
+
+    // per-lane LDS offsets (elements) that do not change from tile to tile
+    const int a_off = pi_row(c_loc) * kPitch + 8 * g;
+    const int t_off = (8 * g + ((lane & 15) >> 2)) * kPitch + ((lane >> 4) & 1) * 16 + 4 * (lane & 3);
+    const int ds_w_off = (wave * 32 + c_loc) * kDsPitch;
+    const int ds_r_off = (8 * (lane >> 4) + ((lane & 15) >> 2)) * kDsPitch + 4 * (lane & 3);
 
     QStage qst, gst;
     float stat_reg = 0.f;
-    auto load_stats = [&](int i0) {
+    auto load_stats = [&](int i0) __attribute__((always_inline)) {
         // threads 0..31 fetch lse (log2 domain, +inf for rows past the end so that P = 0),
         // threads 32..63 fetch delta
         if (threadIdx.x < 64) {
@@ -162,7 +184,7 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
                 stat_reg = i < a.sq ? delta_base[i] : 0.f;
         }
     };
-    auto store_stats = [&](int buf) {
+    auto store_stats = [&](int buf) __attribute__((always_inline)) {
         if (threadIdx.x < 64) stat_lds[buf * 64 + threadIdx.x] = stat_reg;
     };
 
@@ -170,13 +192,17 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
         qst.load(q_base, a.qs[1], t_lo * kBwdBM, a.sq, a.d);
         gst.load(g_base, a.os[1], t_lo * kBwdBM, a.sq, a.d);
         load_stats(t_lo * kBwdBM);
+        qst.fix(t_lo * kBwdBM, a.sq, a.d);
+        gst.fix(t_lo * kBwdBM, a.sq, a.d);
         qst.store(q_lds);
         gst.store(g_lds);
         store_stats(0);
     }
     __syncthreads();
 
+    TSTAMP();
     for (int t = t_lo; t < t_hi; ++t) {
+        TSTAMP();
         const int buf = (t - t_lo) & 1;
         const T* qt = q_lds + buf * SM::kQTile;
         const T* gt = g_lds + buf * SM::kQTile;
@@ -193,7 +219,7 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
 
         const int i_last = min(i0 + kBwdBM, a.sq) - 1;
         // wavefront-uniform activity of each 32-key slab of this workgroup for this query tile
-        auto slab_active = [&](int w) {
+        auto slab_active = [&](int w) __attribute__((always_inline)) {
             const int ks0 = k0 + 32 * w;
             if (ks0 >= a.sk) return false;
             if (a.causal && ks0 > i_last) return false;
@@ -202,22 +228,21 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
         };
         const bool active = slab_active(wave);
 
-        if (active) {
+        auto tile_body = [&](auto mask_tag) __attribute__((always_inline)) {
+            constexpr bool kMask = decltype(mask_tag)::value;
             // ---- S = Q K^T, dP = dO V^T ----
             f32x16_t s_acc, p_acc;
 #pragma unroll
             for (int r = 0; r < 16; ++r) s_acc[r] = 0.f, p_acc[r] = 0.f;
             {
-                const T* qrow = qt + pi_row(c_loc) * kPitch + 8 * g;
-                const T* grow = gt + pi_row(c_loc) * kPitch + 8 * g;
+                const T* qrow = qt + a_off;
+                const T* grow = gt + a_off;
 #pragma unroll
                 for (int x = 0; x < DK; ++x) {
                     s_acc = Mma<T>::mma32(lds_frag<T>(qrow + 16 * x), kf[x], s_acc);
                     p_acc = Mma<T>::mma32(lds_frag<T>(grow + 16 * x), vf[x], p_acc);
                 }
             }
-            const bool need_mask = (kw0 + 32 > a.sk) || (a.causal && kw0 + 31 > i0) ||
-                                   (a.window > 0 && i_last - kw0 >= a.window);
             // ---- P and dS ----
             uint32_t pw[8], dw[8];
 #pragma unroll
@@ -229,8 +254,8 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const int i = i0 + qoff + e;
-                    float s = __builtin_fmaf(s_acc[4 * r4 + e], a.scale_log2, -lse4[e]);
-                    if (a.has_bias) {
+                    float s = __builtin_fmaf(s_acc[4 * r4 + e], c_log2, -lse4[e]);
+                    if constexpr (kBias) {
                         if (bias_per_key)
                             s += bias_k;
                         else if (i < a.sq && key < a.sk)
@@ -238,10 +263,12 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
                                         (int64_t)key * a.bs[3]] * kLog2e;
                     }
                     float p = fast_exp2(s);
-                    if (need_mask && !key_visible(a, i, key)) p = 0.f;
+                    if constexpr (kMask) {
+                        if (!key_visible(a, i, key)) p = 0.f;
+                    }
                     float dp = p_acc[4 * r4 + e];
                     float pd = p;
-                    if (a.dropout) {
+                    if constexpr (kDropout) {
                         float keep = 0.f;
                         if (i < a.sq && key < a.sk) {
                             const uint64_t el =
@@ -265,7 +292,7 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
                 dw[2 * r4 + 1] = pack2<T>(dv[2], dv[3]);
                 // dS^T slab for the dQ pass: row = key (local), columns = 4 consecutive queries
                 u32x2_t w2 = {dw[2 * r4], dw[2 * r4 + 1]};
-                *reinterpret_cast<u32x2_t*>(dst + (wave * 32 + c_loc) * kDsPitch + qoff) = w2;
+                *reinterpret_cast<u32x2_t*>(dst + ds_w_off + qoff) = w2;
             }
             // ---- dV^T += dO^T P,  dK^T += Q^T dS ----
 #pragma unroll
@@ -274,8 +301,7 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
                 u32x4_t dq4 = {dw[4 * hh], dw[4 * hh + 1], dw[4 * hh + 2], dw[4 * hh + 3]};
                 const frag_t pf = __builtin_bit_cast(frag_t, pq);
                 const frag_t df = __builtin_bit_cast(frag_t, dq4);
-                const int off = (16 * hh + 8 * g + ((lane & 15) >> 2)) * kPitch +
-                                ((lane >> 4) & 1) * 16 + 4 * (lane & 3);
+                const int off = 16 * hh * kPitch + t_off;
 #pragma unroll
                 for (int x = 0; x < DV; ++x) {
                     dv_acc[x] =
@@ -284,15 +310,28 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
                         Mma<T>::mma32(lds_frag_tr<T>(qt + off + 32 * x, kPitch), df, dk_acc[x]);
                 }
             }
+        };
+        if (active) {
+            const bool need_mask = (kw0 + 32 > a.sk) || (a.causal && kw0 + 31 > i0) ||
+                                   (a.window > 0 && i_last - kw0 >= a.window);
+            if (need_mask)
+                tile_body(std::true_type{});
+            else
+                tile_body(std::false_type{});
         }
 
+        TSTAMP();
         // stage the next query tile (its buffer was last read before the previous barrier)
         if (have_next) {
+            qst.fix(i0 + kBwdBM, a.sq, a.d);
+            gst.fix(i0 + kBwdBM, a.sq, a.d);
             qst.store(q_lds + (buf ^ 1) * SM::kQTile);
             gst.store(g_lds + (buf ^ 1) * SM::kQTile);
             store_stats(buf ^ 1);
         }
+        TSTAMP();
         __syncthreads();
+        TSTAMP();
 
         // ---- dQ tile = dS K over all active key slabs of the workgroup ----
         {
@@ -310,8 +349,7 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
                 for (int st = 0; st < kBwdWaves; ++st) {
                     if (!slab_active(st)) continue;
                     any = true;
-                    const T* src =
-                        dst + (32 * st + 8 * beta + (n16 >> 2)) * kDsPitch + 4 * (lane & 3);
+                    const T* src = dst + 32 * st * kDsPitch + ds_r_off;
 #pragma unroll
                     for (int qb = 0; qb < 2; ++qb)
                         acc[qb] = Mma<T>::mma16(lds_frag_tr<T>(src + 16 * qb, kDsPitch),
@@ -333,6 +371,7 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
         }
     }
 
+    TSTAMP();
     // ---- write dK, dV ----
     if (key < a.sk) {
         T* dk_row = reinterpret_cast<T*>(a.dk) + b * a.dks[0] + (int64_t)key * a.dks[1] + h * a.dks[2];
@@ -355,39 +394,58 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
     }
 }
 
-template <typename T, int DPAD>
-int launch_bwd(const AttnArgs& a, hipStream_t st) {
+template <typename T, int DPAD, bool kBias, bool kDropout>
+int launch(const AttnArgs& a, hipStream_t st) {
     typedef BwdSmem<T, DPAD> SM;
     const size_t smem = SM::kBytes;
     const int n_kt = (a.sk + kBwdBN - 1) / kBwdBN;
     const int64_t blocks = (int64_t)n_kt * a.batch * a.heads;
     if (blocks <= 0 || blocks > 0x7FFFFFFF) return SLAPO_ERR_SHAPE;
-    auto kern = attn_bwd_kernel<T, DPAD>;
+    auto kern = attn_bwd_kernel<T, DPAD, kBias, kDropout>;
     if (smem > 48 * 1024) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)smem) != hipSuccess)
-            return SLAPO_ERR_LAUNCH;
+        static bool raised = false;  // per instantiation
+        if (!raised) {
+            if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)smem) != hipSuccess)
+                return SLAPO_ERR_LAUNCH;
+            raised = true;
+        }
     }
+#ifdef EXP_OCC
+    {
+        static bool once = false;
+        if (!once) {
+            once = true;
+            int nb = -1;
+            hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, reinterpret_cast<const void*>(kern), kBwdThreads, smem);
+            hipFuncAttributes fa;
+            hipFuncGetAttributes(&fa, reinterpret_cast<const void*>(kern));
+            fprintf(stderr, "[occ] %s DPAD=%d smem=%zu regs=%d staticsmem=%zu maxthreads=%d -> blocks/CU=%d\n", __func__, DPAD, smem, fa.numRegs, fa.sharedSizeBytes, fa.maxThreadsPerBlock, nb);
+        }
+    }
+#endif
     hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kBwdThreads), smem, st, a);
     return check_launch();
 }
 
+template <typename T, int DPAD>
+int dispatch_flags(const AttnArgs& a, hipStream_t st) {
+    if (a.has_bias) {
+        if (a.dropout) return launch<T, DPAD, true, true>(a, st);
+        return launch<T, DPAD, true, false>(a, st);
+    }
+    if (a.dropout) return launch<T, DPAD, false, true>(a, st);
+    return launch<T, DPAD, false, false>(a, st);
+}
+
 template <typename T>
-int dispatch_bwd(const AttnArgs& a, hipStream_t st) {
-    if (a.d <= 32) return launch_bwd<T, 32>(a, st);
-    if (a.d <= 64) return launch_bwd<T, 64>(a, st);
-    if (a.d <= 96) return launch_bwd<T, 96>(a, st);
-    if (a.d <= 128) return launch_bwd<T, 128>(a, st);
+int dispatch(const AttnArgs& a, hipStream_t st) {
+    if (a.d <= 64) return dispatch_flags<T, 64>(a, st);
+    if (a.d <= 96) return dispatch_flags<T, 96>(a, st);
+    if (a.d <= 128) return dispatch_flags<T, 128>(a, st);
     return SLAPO_ERR_SHAPE;
 }
 
-}  // namespace
-
-namespace slapo {
-int attn_bwd_mfma(const AttnArgs& a, int dtype, hipStream_t st) {
-    if (dtype == SLAPO_F16) return dispatch_bwd<f16_t>(a, st);
-    if (dtype == SLAPO_BF16) return dispatch_bwd<bf16_t>(a, st);
-    return SLAPO_ERR_DTYPE;
-}
+}  // namespace bwd
 }  // namespace slapo

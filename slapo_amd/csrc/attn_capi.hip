@@ -4,8 +4,10 @@
 #include "attn_common.h"
 
 namespace slapo {
-int attn_fwd_mfma(const AttnArgs& a, int dtype, hipStream_t st);
-int attn_bwd_mfma(const AttnArgs& a, int dtype, hipStream_t st);
+int attn_fwd_mfma_f16(const AttnArgs& a, hipStream_t st);
+int attn_fwd_mfma_bf16(const AttnArgs& a, hipStream_t st);
+int attn_bwd_mfma_f16(const AttnArgs& a, hipStream_t st);
+int attn_bwd_mfma_bf16(const AttnArgs& a, hipStream_t st);
 int attn_fwd_f32(const AttnArgs& a, hipStream_t st);
 int attn_bwd_f32(const AttnArgs& a, hipStream_t st);
 }  // namespace slapo
@@ -154,6 +156,14 @@ bool half_ptrs_ok(std::initializer_list<const void*> ptrs) {
 
 }  // namespace
 
+#ifdef EXP_TIMING
+void* g_timing_buf = nullptr;
+extern "C" int slapo_dbg_timing(unsigned long long* out, int n) {
+    hipDeviceSynchronize();
+    return (int)hipMemcpy(out, g_timing_buf, n * 8, hipMemcpyDeviceToHost);
+}
+#endif
+
 extern "C" int slapo_amd_attn_fwd(const slapo_attn_params* prm, const void* q, const void* k,
                                   const void* v, const float* bias, void* o, float* lse,
                                   void* stream) {
@@ -164,9 +174,15 @@ extern "C" int slapo_amd_attn_fwd(const slapo_attn_params* prm, const void* q, c
     a.q = q, a.k = k, a.v = v, a.o = o, a.lse = lse;
     set_bias(&a, bias);
     hipStream_t st = (hipStream_t)stream;
+#ifdef EXP_TIMING
+    {
+        if (!g_timing_buf) { hipMalloc(&g_timing_buf, 1 << 16); hipMemset(g_timing_buf, 0, 1 << 16); }
+        a.delta = (float*)g_timing_buf;
+    }
+#endif
     if (prm->dtype == SLAPO_F32) return attn_fwd_f32(a, st);
     if (!half_ptrs_ok({q, k, v, o})) return SLAPO_ERR_ALIGN;
-    return attn_fwd_mfma(a, prm->dtype, st);
+    return prm->dtype == SLAPO_F16 ? attn_fwd_mfma_f16(a, st) : attn_fwd_mfma_bf16(a, st);
 }
 
 extern "C" size_t slapo_amd_attn_bwd_workspace_bytes(const slapo_attn_params* prm) {
@@ -251,7 +267,11 @@ extern "C" int slapo_amd_attn_bwd_stages(const slapo_attn_params* prm, const voi
     }
     if (stages & SLAPO_BWD_MAIN) {
         a.dq = dq_acc;
-        rc = attn_bwd_mfma(a, prm->dtype, st);
+#ifdef EXP_TIMING
+        if (!g_timing_buf) { hipMalloc(&g_timing_buf, 1 << 16); hipMemset(g_timing_buf, 0, 1 << 16); }
+        a.o = g_timing_buf;
+#endif
+        rc = prm->dtype == SLAPO_F16 ? attn_bwd_mfma_f16(a, st) : attn_bwd_mfma_bf16(a, st);
         if (rc != SLAPO_OK) return rc;
     }
     if (stages & SLAPO_BWD_FINISH) {

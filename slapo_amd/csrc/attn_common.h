@@ -82,16 +82,38 @@ __device__ __forceinline__ constexpr int acc_row(int r, int g) {
     return ((r >> 3) << 4) + (g << 3) + (((r >> 2) & 1) << 2) + (r & 3);
 }
 
+// Two floats -> one packed register of T, round to nearest even (v_cvt_pk_{f16,bf16}_f32).
 template <typename T>
 __device__ __forceinline__ uint32_t pack2(float a, float b) {
     typedef T pair_t __attribute__((ext_vector_type(2)));
-    pair_t p = {(T)a, (T)b};
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    f32x2_t v = {a, b};
+    pair_t p = __builtin_convertvector(v, pair_t);
     return __builtin_bit_cast(uint32_t, p);
 }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-__device__ __forceinline__ float xor32(float v) { return __shfl_xor(v, 32, 64); }
+// Exchange with lane l ^ 32 through v_permlane32_swap (upper half of the first register <-> lower
+// half of the second).  Starting from two copies of v, the first register ends up holding the lower
+// half's values on all lanes and the second the upper half's.  Written as inline assembly, with the
+// wait states the instruction needs after a VALU write of its operands.
+__device__ __forceinline__ void swap32(float v, float& lo_val, float& hi_val) {
+    float a = v, b = v;
+    asm volatile("s_nop 1\n\tv_permlane32_swap_b32 %0, %1\n\ts_nop 1" : "+v"(a), "+v"(b));
+    lo_val = a;
+    hi_val = b;
+}
+__device__ __forceinline__ float max_xor32(float v) {
+    float a, b;
+    swap32(v, a, b);
+    return fmaxf(a, b);
+}
+__device__ __forceinline__ float sum_xor32(float v) {
+    float a, b;
+    swap32(v, a, b);
+    return a + b;
+}
 
 // Kernel argument block (filled by the host dispatcher from slapo_attn_params).
 struct AttnArgs {
@@ -133,7 +155,10 @@ __device__ __forceinline__ void query_range(const AttnArgs& a, int k_lo, int k_h
     i_hi = a.window > 0 ? min(a.sq, k_hi - 1 + a.window) : a.sq;
 }
 
-// Stage a [64 x DPAD] tile of T (rows row0.., zero beyond n_rows / beyond d) through registers.
+// Stage a [ROWS x DPAD] tile of T (rows row0.., zero beyond n_rows / beyond d) through registers.
+// The global loads are unconditional (out-of-range rows are clamped to the last valid row and
+// zeroed when the tile is written to LDS), so they stay in the caller's basic block and the
+// compiler can leave them in flight across the math that follows.
 template <typename T, int DPAD, int ROWS, int THREADS>
 struct TileStage {
     static constexpr int kChunksPerRow = DPAD / 8;
@@ -149,11 +174,21 @@ struct TileStage {
             const int c = threadIdx.x + u * THREADS;
             const int row = c / kChunksPerRow;
             const int cc = c % kChunksPerRow;
-            const int gr = row0 + row;
-            u32x4_t v = {0u, 0u, 0u, 0u};
-            if ((kChunks % THREADS == 0 || c < kChunks) && gr < n_rows && cc * 8 < d)
-                v = *reinterpret_cast<const u32x4_t*>(base + (int64_t)gr * row_stride + cc * 8);
-            r[u] = v;
+            const int gr = min(row0 + row, n_rows - 1);
+            if (kChunks % THREADS == 0 || c < kChunks)
+                r[u] = *reinterpret_cast<const u32x4_t*>(base + (int64_t)gr * row_stride +
+                                                         min(cc * 8, d - 8));
+        }
+    }
+    // Zero what `load` clamped: rows past n_rows and columns past d.
+    __device__ __forceinline__ void fix(int row0, int n_rows, int d) {
+        if (row0 + ROWS <= n_rows && d == DPAD) return;  // uniform: whole tile valid
+#pragma unroll
+        for (int u = 0; u < kPerThread; ++u) {
+            const int c = threadIdx.x + u * THREADS;
+            const int row = c / kChunksPerRow;
+            const int cc = c % kChunksPerRow;
+            if (row0 + row >= n_rows || cc * 8 >= d) r[u] = u32x4_t{0u, 0u, 0u, 0u};
         }
     }
     __device__ __forceinline__ void store(T* lds) const {
