@@ -17,8 +17,10 @@ using namespace slapo;
 namespace {
 
 // delta[bh, i] = sum_d dO[b,i,h,d] * O[b,i,h,d]; eight lanes share a row, 16 bytes per lane.
+// When zero_acc is given, the same lanes also clear row (bh, i) of the fp32 dQ accumulator, so the
+// backward needs one preparation launch instead of two.
 template <typename T>
-__global__ __launch_bounds__(256) void attn_delta_kernel(const AttnArgs a) {
+__global__ __launch_bounds__(256) void attn_delta_kernel(const AttnArgs a, float* zero_acc) {
     constexpr int V = Elem<T>::kPerVec;
     const int64_t row = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 3;
     const int sub = threadIdx.x & 7;
@@ -40,6 +42,11 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const AttnArgs a) {
                 acc = __builtin_fmaf(Elem<T>::to_f32(po.v[e]), Elem<T>::to_f32(pg.v[e]), acc);
         }
     }
+    if (zero_acc && row < n_rows) {
+        float* z = zero_acc + row * a.d;
+        for (int c = sub * 4; c < a.d; c += 32)
+            *reinterpret_cast<f32x4_t*>(z + c) = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    }
     acc += __shfl_xor(acc, 1, 64);
     acc += __shfl_xor(acc, 2, 64);
     acc += __shfl_xor(acc, 4, 64);
@@ -60,11 +67,6 @@ __global__ __launch_bounds__(256) void attn_delta_scalar_kernel(const AttnArgs a
     float acc = 0.f;
     for (int e = 0; e < a.d; ++e) acc = __builtin_fmaf(o[e], g[e], acc);
     a.delta[row] = acc;
-}
-
-__global__ __launch_bounds__(256) void fill_zero_kernel(f32x4_t* p, int64_t n4) {
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i < n4) p[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 }
 
 // dq[b,i,h,:] = T(scale * dq_acc[bh,i,:]);  8 lanes per row, 4 floats per lane per trip.
@@ -234,7 +236,8 @@ extern "C" int slapo_amd_attn_bwd_stages(const slapo_attn_params* prm, const voi
                                 strides_ok(prm->o_strides, 4);
             if (vec_ok) {
                 const unsigned blocks = (unsigned)((rows * 8 + 255) / 256);
-                hipLaunchKernelGGL((attn_delta_kernel<float>), dim3(blocks), dim3(256), 0, st, a);
+                hipLaunchKernelGGL((attn_delta_kernel<float>), dim3(blocks), dim3(256), 0, st, a,
+                                   (float*)nullptr);
             } else {
                 const unsigned blocks = (unsigned)((rows + 255) / 256);
                 hipLaunchKernelGGL(attn_delta_scalar_kernel, dim3(blocks), dim3(256), 0, st, a);
@@ -255,13 +258,13 @@ extern "C" int slapo_amd_attn_bwd_stages(const slapo_attn_params* prm, const voi
 
     const unsigned row_blocks = (unsigned)((rows * 8 + 255) / 256);
     if (stages & SLAPO_BWD_PREPARE) {
+        // head_dim % 8 == 0, so each accumulator row is a whole number of 16-byte stores
         if (prm->dtype == SLAPO_F16)
-            hipLaunchKernelGGL((attn_delta_kernel<f16_t>), dim3(row_blocks), dim3(256), 0, st, a);
+            hipLaunchKernelGGL((attn_delta_kernel<f16_t>), dim3(row_blocks), dim3(256), 0, st, a,
+                               dq_acc);
         else
-            hipLaunchKernelGGL((attn_delta_kernel<bf16_t>), dim3(row_blocks), dim3(256), 0, st, a);
-        const int64_t n4 = rows * a.d / 4;  // head_dim % 8 == 0
-        hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((n4 + 255) / 256)), dim3(256), 0, st,
-                           reinterpret_cast<f32x4_t*>(dq_acc), n4);
+            hipLaunchKernelGGL((attn_delta_kernel<bf16_t>), dim3(row_blocks), dim3(256), 0, st, a,
+                               dq_acc);
         rc = check_launch();
         if (rc != SLAPO_OK) return rc;
     }

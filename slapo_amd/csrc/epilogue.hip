@@ -48,8 +48,12 @@ __device__ __forceinline__ Chunk<T, V> load_chunk(const T* p) {
         c.v[0] = *p;
     } else {
         static_assert(sizeof(Chunk<T, V>) == 16, "vector chunk must be 16 bytes");
+#ifdef EPI_NO_NT
+        *reinterpret_cast<u32x4_t*>(&c) = *reinterpret_cast<const u32x4_t*>(p);
+#else
         *reinterpret_cast<u32x4_t*>(&c) =
             __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(p));
+#endif
     }
     return c;
 }
@@ -68,8 +72,12 @@ __device__ __forceinline__ void store_chunk(T* p, const Chunk<T, V>& c) {
     if constexpr (V == 1) {
         *p = c.v[0];
     } else {
+#ifdef EPI_NO_NT_ST
+        *reinterpret_cast<u32x4_t*>(p) = *reinterpret_cast<const u32x4_t*>(&c);
+#else
         __builtin_nontemporal_store(*reinterpret_cast<const u32x4_t*>(&c),
                                     reinterpret_cast<u32x4_t*>(p));
+#endif
     }
 }
 
@@ -92,7 +100,10 @@ __device__ __forceinline__ uint32_t keep_bits(const DropoutState& s, uint64_t e0
 // ----------------------------------------------------------------------------------------
 // Forward kernels: flat over chunks; a block covers kUnroll * 256 consecutive chunks.
 // ----------------------------------------------------------------------------------------
-constexpr int kUnroll = 4;
+#ifndef EPI_UNROLL
+#define EPI_UNROLL 1
+#endif
+constexpr int kUnroll = EPI_UNROLL;
 
 template <typename T, int V>
 __global__ __launch_bounds__(256) void bias_gelu_fwd_kernel(const T* __restrict__ y,
@@ -167,7 +178,10 @@ __global__ __launch_bounds__(256) void bias_dropout_residual_fwd_kernel(
 // keeping per-thread fp32 column sums; the 4 row-lanes are combined through LDS and written
 // as one fp32 partial row per block.
 // ----------------------------------------------------------------------------------------
-constexpr int kRowsPerBlock = 64;
+#ifndef EPI_ROWS
+#define EPI_ROWS 64
+#endif
+constexpr int kRowsPerBlock = EPI_ROWS;
 constexpr int kRowLanes = 4;
 constexpr int kColLanes = 64;
 
@@ -263,15 +277,33 @@ __global__ __launch_bounds__(256) void bias_dropout_bwd_kernel(const T* __restri
                       });
 }
 
+// Second stage of the column reduction: a block owns 64 columns; its 4 row-lanes walk the partial
+// rows with a stride of 4 (coalesced 256-byte reads), then combine through LDS.
 template <typename T>
 __global__ __launch_bounds__(256) void colsum_finish_kernel(const float* __restrict__ partial,
                                                             T* __restrict__ dbias,
                                                             int64_t n_partials, int64_t cols) {
-    const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (c >= cols) return;
+    __shared__ float red[kRowLanes][kColLanes];
+    const int cx = threadIdx.x % kColLanes;
+    const int ry = threadIdx.x / kColLanes;
+    const int64_t c = (int64_t)blockIdx.x * kColLanes + cx;
     float t = 0.f;
-    for (int64_t k = 0; k < n_partials; ++k) t += partial[k * cols + c];
-    dbias[c] = Elem<T>::from_f32(t);
+    if (c < cols) {
+        float t0 = 0.f, t1 = 0.f, t2 = 0.f, t3 = 0.f;
+        int64_t k = ry;
+        for (; k + 3 * kRowLanes < n_partials; k += 4 * kRowLanes) {
+            t0 += partial[k * cols + c];
+            t1 += partial[(k + kRowLanes) * cols + c];
+            t2 += partial[(k + 2 * kRowLanes) * cols + c];
+            t3 += partial[(k + 3 * kRowLanes) * cols + c];
+        }
+        for (; k < n_partials; k += kRowLanes) t0 += partial[k * cols + c];
+        t = (t0 + t1) + (t2 + t3);
+    }
+    red[ry][cx] = t;
+    __syncthreads();
+    if (ry == 0 && c < cols)
+        dbias[c] = Elem<T>::from_f32((red[0][cx] + red[1][cx]) + (red[2][cx] + red[3][cx]));
 }
 
 // ----------------------------------------------------------------------------------------
@@ -362,7 +394,7 @@ inline bool bwd_grid(int64_t rows, int64_t cols, int v, dim3* grid) {
 template <typename T>
 int finish_colsum(const float* partial, void* dbias, int64_t rows, int64_t cols, hipStream_t st) {
     const int64_t n_partials = (rows + kRowsPerBlock - 1) / kRowsPerBlock;
-    const unsigned blocks = (unsigned)((cols + 255) / 256);
+    const unsigned blocks = (unsigned)((cols + kColLanes - 1) / kColLanes);
     hipLaunchKernelGGL((colsum_finish_kernel<T>), dim3(blocks), dim3(256), 0, st, partial,
                        (T*)dbias, n_partials, cols);
     return check_launch();
