@@ -90,9 +90,12 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
     int tcount = 0;
     const bool trec = (blockIdx.x == EXP_TIMING) && threadIdx.x == 0;
 #define TSTAMP() do { if (trec) tbuf[tcount++] = __builtin_readcyclecounter(); } while (0)
+// stamp taken only after `dep` has been produced (forces the wait for the MFMA / VALU results)
+#define TSTAMP2(dep) do { float dd = (dep); asm volatile("" :: "v"(dd)); if (trec) tbuf[tcount++] = __builtin_readcyclecounter(); } while (0)
     TSTAMP();
 #else
 #define TSTAMP() do {} while (0)
+#define TSTAMP2(dep) do {} while (0)
 #endif
     const int kw0 = k0 + wave * 32;
     const int key = kw0 + c_loc;  // this lane's key column
@@ -172,20 +175,20 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
     const int ds_r_off = (8 * (lane >> 4) + ((lane & 15) >> 2)) * kDsPitch + 4 * (lane & 3);
 
     QStage qst, gst;
+    // lse / delta of a query tile: threads 0..31 fetch lse, threads 32..63 delta.  The load is
+    // unconditional (row clamped) and its result is not touched until the tile is written to LDS.
     float stat_reg = 0.f;
+    const float* stat_src = (threadIdx.x < 32) ? lse_base : delta_base;
     auto load_stats = [&](int i0) __attribute__((always_inline)) {
-        // threads 0..31 fetch lse (log2 domain, +inf for rows past the end so that P = 0),
-        // threads 32..63 fetch delta
-        if (threadIdx.x < 64) {
-            const int i = i0 + (threadIdx.x & 31);
-            if (threadIdx.x < 32)
-                stat_reg = i < a.sq ? lse_base[i] * kLog2e : INFINITY;
-            else
-                stat_reg = i < a.sq ? delta_base[i] : 0.f;
-        }
+        if (threadIdx.x < 64) stat_reg = stat_src[min(i0 + (int)(threadIdx.x & 31), a.sq - 1)];
     };
-    auto store_stats = [&](int buf) __attribute__((always_inline)) {
-        if (threadIdx.x < 64) stat_lds[buf * 64 + threadIdx.x] = stat_reg;
+    auto store_stats = [&](int buf, int i0) __attribute__((always_inline)) {
+        if (threadIdx.x < 64) {
+            const bool ok = i0 + (int)(threadIdx.x & 31) < a.sq;
+            // lse in log2 units, +inf for rows past the end so that P = 0 there; delta 0
+            float v = (threadIdx.x < 32) ? (ok ? stat_reg * kLog2e : INFINITY) : (ok ? stat_reg : 0.f);
+            stat_lds[buf * 64 + threadIdx.x] = v;
+        }
     };
 
     if (t_lo < t_hi) {
@@ -196,13 +199,70 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
         gst.fix(t_lo * kBwdBM, a.sq, a.d);
         qst.store(q_lds);
         gst.store(g_lds);
-        store_stats(0);
+        store_stats(0, t_lo * kBwdBM);
     }
     __syncthreads();
 
+    // wavefront-uniform activity of 32-key slab w of this workgroup for the query tile at i0
+    auto slab_active = [&](int w, int i0) __attribute__((always_inline)) {
+        const int ks0 = k0 + 32 * w;
+        const int i_last = min(i0 + kBwdBM, a.sq) - 1;
+        if (ks0 >= a.sk) return false;
+        if (a.causal && ks0 > i_last) return false;
+        if (a.window > 0 && i0 - (ks0 + 31) >= a.window) return false;
+        return true;
+    };
+
+    // dQ tile = dS K over all active key slabs of the workgroup, for the query tile at i0 whose
+    // dS^T sits in `dst`; added to the fp32 accumulator with hardware atomics.
+    auto dq_phase = [&](const T* dst, int i0) __attribute__((always_inline)) {
+        const int beta = lane >> 4;
+        const int n16 = lane & 15;
+#pragma unroll
+        for (int nb = 0; nb < NDB; ++nb) {
+            const int blk = wave + nb * kBwdWaves;
+            if (blk >= NBLK) continue;
+            f32x4_t acc[2];
+#pragma unroll
+            for (int qb = 0; qb < 2; ++qb) acc[qb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+            bool any = false;
+#pragma unroll
+            for (int st = 0; st < kBwdWaves; ++st) {
+                if (!slab_active(st, i0)) continue;
+                any = true;
+                const T* src = dst + 32 * st * kDsPitch + ds_r_off;
+#pragma unroll
+                for (int qb = 0; qb < 2; ++qb)
+                    acc[qb] = Mma<T>::mma16(lds_frag_tr<T>(src + 16 * qb, kDsPitch), ktf[nb][st],
+                                            acc[qb]);
+            }
+            if (!any) continue;
+            const int dcol = 16 * blk + n16;
+            float* dq_col = dq_base + (int64_t)(i0 + 4 * beta) * a.d + dcol;
+            if (i0 + kBwdBM <= a.sq && dcol < a.d) {
+#pragma unroll
+                for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        unsafeAtomicAdd(dq_col + (int64_t)(16 * qb + r) * a.d, acc[qb][r]);
+            } else if (dcol < a.d) {
+#pragma unroll
+                for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        if (i0 + 16 * qb + 4 * beta + r < a.sq)
+                            unsafeAtomicAdd(dq_col + (int64_t)(16 * qb + r) * a.d, acc[qb][r]);
+            }
+        }
+    };
+
     TSTAMP();
-    for (int t = t_lo; t < t_hi; ++t) {
+    // Iteration t: request tile t+1, run the dQ phase of tile t-1 (its dS^T was completed before the
+    // last barrier), then the S / dP / dV / dK work of tile t, then write tile t+1 to LDS.
+    // One extra trip drains the dQ phase of the last tile.
+    for (int t = t_lo; t <= t_hi; ++t) {
         TSTAMP();
+        const bool compute = t < t_hi;
         const int buf = (t - t_lo) & 1;
         const T* qt = q_lds + buf * SM::kQTile;
         const T* gt = g_lds + buf * SM::kQTile;
@@ -216,17 +276,10 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
             gst.load(g_base, a.os[1], i0 + kBwdBM, a.sq, a.d);
             load_stats(i0 + kBwdBM);
         }
+        if (t > t_lo) dq_phase(ds_lds + (buf ^ 1) * SM::kDsTile, i0 - kBwdBM);
 
         const int i_last = min(i0 + kBwdBM, a.sq) - 1;
-        // wavefront-uniform activity of each 32-key slab of this workgroup for this query tile
-        auto slab_active = [&](int w) __attribute__((always_inline)) {
-            const int ks0 = k0 + 32 * w;
-            if (ks0 >= a.sk) return false;
-            if (a.causal && ks0 > i_last) return false;
-            if (a.window > 0 && i0 - (ks0 + 31) >= a.window) return false;
-            return true;
-        };
-        const bool active = slab_active(wave);
+        const bool active = compute && slab_active(wave, i0);
 
         auto tile_body = [&](auto mask_tag) __attribute__((always_inline)) {
             constexpr bool kMask = decltype(mask_tag)::value;
@@ -327,48 +380,11 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
             gst.fix(i0 + kBwdBM, a.sq, a.d);
             qst.store(q_lds + (buf ^ 1) * SM::kQTile);
             gst.store(g_lds + (buf ^ 1) * SM::kQTile);
-            store_stats(buf ^ 1);
+            store_stats(buf ^ 1, i0 + kBwdBM);
         }
         TSTAMP();
-        __syncthreads();
+        if (compute) __syncthreads();
         TSTAMP();
-
-        // ---- dQ tile = dS K over all active key slabs of the workgroup ----
-        {
-            const int beta = lane >> 4;
-            const int n16 = lane & 15;
-#pragma unroll
-            for (int nb = 0; nb < NDB; ++nb) {
-                const int blk = wave + nb * kBwdWaves;
-                if (blk >= NBLK) continue;
-                f32x4_t acc[2];
-#pragma unroll
-                for (int qb = 0; qb < 2; ++qb) acc[qb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-                bool any = false;
-#pragma unroll
-                for (int st = 0; st < kBwdWaves; ++st) {
-                    if (!slab_active(st)) continue;
-                    any = true;
-                    const T* src = dst + 32 * st * kDsPitch + ds_r_off;
-#pragma unroll
-                    for (int qb = 0; qb < 2; ++qb)
-                        acc[qb] = Mma<T>::mma16(lds_frag_tr<T>(src + 16 * qb, kDsPitch),
-                                                ktf[nb][st], acc[qb]);
-                }
-                if (!any) continue;
-                const int dcol = 16 * blk + n16;
-                if (dcol < a.d) {
-#pragma unroll
-                    for (int qb = 0; qb < 2; ++qb)
-#pragma unroll
-                        for (int r = 0; r < 4; ++r) {
-                            const int i = i0 + 16 * qb + 4 * beta + r;
-                            if (i < a.sq)
-                                unsafeAtomicAdd(dq_base + (int64_t)i * a.d + dcol, acc[qb][r]);
-                        }
-                }
-            }
-        }
     }
 
     TSTAMP();

@@ -323,6 +323,9 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_fwd_kerne
                                                : finish_scores(s_a, t_lo, std::false_type{});
         update_reference(mx);
     }
+    // K slot 0 is overwritten (with tile 2) at the end of iteration 0: every wavefront must have
+    // finished reading it for the scores above before any wavefront gets there.
+    __syncthreads();
 
     // iteration r: requests tile r+3 into (k_ld, v_ld), writes tile r+2 from (k_st, v_st)
     auto iteration = [&](int r, f32x16_t (&s_cur)[2], f32x16_t (&s_next)[2], Stage& k_ld,
