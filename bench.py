@@ -91,10 +91,10 @@ class AttentionStep:
         self.backward(self._lib_mod.BWD_PREPARE)
         if ev is not None:
             ev[0].record()
-        self.backward(self._lib_mod.BWD_MAIN)
+        self.backward(self._lib_mod.BWD_DKDV)
         if ev is not None:
             ev[1].record()
-        self.backward(self._lib_mod.BWD_FINISH)
+        self.backward(self._lib_mod.BWD_DQ)
 
 
 def bench_epilogues(device, iters=40):

@@ -164,7 +164,7 @@ typedef struct slapo_attn_params {
 int slapo_amd_attn_fwd(const slapo_attn_params* prm, const void* q, const void* k, const void* v,
                        const float* bias, void* o, float* lse, void* stream);
 
-/* Workspace (bytes) the backward needs: fp32 dQ accumulator + fp32 delta = rowsum(dO * O). */
+/* Workspace (bytes) the backward needs: fp32 delta = rowsum(dO * O), one value per query row. */
 size_t slapo_amd_attn_bwd_workspace_bytes(const slapo_attn_params* prm);
 
 /* dq/dk/dv use q_strides/k_strides/v_strides of a DENSE [B,S,H,D] layout given in
@@ -175,16 +175,18 @@ int slapo_amd_attn_bwd(const slapo_attn_params* prm, const void* q, const void* 
                        const int64_t dk_strides[3], const int64_t dv_strides[3], void* workspace,
                        size_t workspace_bytes, void* stream);
 
-/* The backward runs as three stages on `stream`: PREPARE (delta = rowsum(dO * O), clear the fp32
- * dQ accumulator), MAIN (the dK / dV / dQ-accumulate kernel) and FINISH (dQ accumulator -> dq in
- * the tensor dtype).  slapo_amd_attn_bwd runs all three; this entry point runs the stages named in
- * `stages` (a bit-or of the constants below) so that a caller can place its own events around one
- * of them or overlap PREPARE with other work.  Arguments are those of slapo_amd_attn_bwd and must
- * be the same across the calls of one backward pass.  For SLAPO_F32 the MAIN stage writes dq
- * directly and FINISH is a no-op. */
+/* The backward runs as three stages on `stream`: PREPARE (delta = rowsum(dO * O) into the
+ * workspace), DKDV (workgroups own key rows and write dk, dv) and DQ (workgroups own query rows
+ * and write dq).  DKDV and DQ both recompute the probabilities from lse, depend only on PREPARE
+ * and write disjoint outputs: no atomics, no zero-initialised accumulator, bitwise reproducible.
+ * slapo_amd_attn_bwd runs all three; this entry point runs the stages named in `stages` (a bit-or
+ * of the constants below) so that a caller can time one of them or put DKDV and DQ on different
+ * streams.  Arguments are those of slapo_amd_attn_bwd and must be the same across the calls of one
+ * backward pass.  For SLAPO_F32 both gradient stages are served by the FMA kernels (DKDV runs
+ * them all, DQ is a no-op). */
 #define SLAPO_BWD_PREPARE 1
-#define SLAPO_BWD_MAIN 2
-#define SLAPO_BWD_FINISH 4
+#define SLAPO_BWD_DKDV 2
+#define SLAPO_BWD_DQ 4
 #define SLAPO_BWD_ALL 7
 int slapo_amd_attn_bwd_stages(const slapo_attn_params* prm, const void* q, const void* k,
                               const void* v, const float* bias, const void* o, const void* dout,

@@ -117,7 +117,7 @@ PROTOTYPES = {
     ),
 }
 
-BWD_PREPARE, BWD_MAIN, BWD_FINISH, BWD_ALL = 1, 2, 4, 7
+BWD_PREPARE, BWD_DKDV, BWD_DQ, BWD_ALL = 1, 2, 4, 7
 
 _lib = None
 _lock = threading.Lock()

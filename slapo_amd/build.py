@@ -42,6 +42,8 @@ PER_FILE_FLAGS = {
     "attn_fwd_bf16.hip": ["-fno-honor-nans"],
     "attn_bwd_f16.hip": ["-fno-honor-nans"],
     "attn_bwd_bf16.hip": ["-fno-honor-nans"],
+    "attn_bwd_dq_f16.hip": ["-fno-honor-nans"],
+    "attn_bwd_dq_bf16.hip": ["-fno-honor-nans"],
 }
 
 

@@ -1,0 +1,7 @@
+// bf16 instantiation of the dQ backward kernel (one translation unit per element type keeps the
+// builds parallel).
+#include "attn_bwd_dq_impl.h"
+
+namespace slapo {
+int attn_bwd_dq_mfma_bf16(const AttnArgs& a, hipStream_t st) { return bwd_dq::dispatch<bf16_t>(a, st); }
+}  // namespace slapo

@@ -1,0 +1,369 @@
+// Flash-attention backward, dQ half, for gfx950 (fp16 / bf16 inputs, fp32 accumulation).
+//
+// The backward is split in two kernels that each recompute the probabilities: this one owns query
+// rows and produces dQ, its sibling owns key rows and produces dK / dV.  Neither needs atomics or
+// a zero-initialised accumulator, and the result does not depend on scheduling order.
+//
+// One workgroup (4 wavefronts) owns 128 consecutive queries of one (batch, head); wavefront w
+// owns 32 of them and keeps their Q^T and dO^T fragments, lse and delta in registers.  Keys and
+// values stream through LDS in tiles of 64, double buffered and staged through registers (the
+// global loads of tile t+1 are in flight while tile t is processed).  Per key tile, lane l = query
+// i, registers = keys:
+//   S^T  = K Q^T, dP^T = V dO^T    A = K / V rows from LDS (row-permuted 128-bit reads)
+//   P^T  = exp2(S^T * scale - lse), dS^T = P^T * (dP^T - delta)
+//   dQ^T += K^T dS^T               B = dS^T straight from the accumulator registers, A = K^T read
+//                                  from the row-major K tile with the transposing LDS read.
+//
+// Reference semantics: autograd of slapo/op/attention.py:163-181 (attention_bmk).
+#pragma once
+#include <type_traits>
+
+#include "attn_common.h"
+
+namespace slapo {
+namespace bwd_dq {
+
+constexpr int kWaves = 4;
+constexpr int kThreads = kWaves * 64;
+constexpr int kBM = kWaves * 32;
+constexpr int kBN = 64;
+constexpr int kKRing = 2;
+constexpr int kVRing = 2;
+
+template <typename T, int DPAD, bool kBias, bool kDropout>
+__global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_dq_kernel(
+    const AttnArgs a) {
+    typedef typename Mma<T>::frag frag_t;
+    typedef TileStage<T, DPAD, kBN, kThreads> Stage;
+    constexpr int kPitch = Stage::kPitch;
+    constexpr int kTileElems = kBN * kPitch;
+    constexpr int DK = DPAD / 16;  // k-steps over the head dimension
+    constexpr int DV = DPAD / 32;  // 32-row blocks of dQ^T
+
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    T* smem = reinterpret_cast<T*>(smem_raw);
+    T* k_lds = smem;                        // K[kKRing][tile]
+    T* v_lds = smem + kKRing * kTileElems;  // V[kVRing][tile]
+
+    const int n_bh = a.batch * a.heads;
+    const int n_qt = (a.sq + kBM - 1) / kBM;
+    const int bh = blockIdx.x % n_bh;
+    const int qt = n_qt - 1 - blockIdx.x / n_bh;  // heaviest (latest) query tiles first
+    const int b = bh / a.heads;
+    const int h = bh % a.heads;
+    const int q0 = qt * kBM;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wavefront-uniform
+    const int g = lane >> 5;
+    const int i_loc = lane & 31;
+    const int wq0 = q0 + wave * 32;
+    const int q_row = wq0 + i_loc;
+
+    const T* q_base = reinterpret_cast<const T*>(a.q) + b * a.qs[0] + h * a.qs[2];
+    const T* k_base = reinterpret_cast<const T*>(a.k) + b * a.ks[0] + h * a.ks[2];
+    const T* v_base = reinterpret_cast<const T*>(a.v) + b * a.vs[0] + h * a.vs[2];
+    const T* g_base = reinterpret_cast<const T*>(a.dout) + b * a.os[0] + h * a.os[2];
+
+    // Q^T and dO^T fragments: column i = this lane's query, k-slots = 8 head-dim elements.
+    frag_t qf[DK], gf[DK];
+    float lse2 = INFINITY;  // log2 units; +inf for rows past the end so that P = 0 there
+    float delta = 0.f;
+    {
+        const int qr = min(q_row, a.sq - 1);
+#pragma unroll
+        for (int t = 0; t < DK; ++t) {
+            const int d0 = 16 * t + 8 * g;
+            const int dc = min(d0, a.d - 8);
+            u32x4_t qv = *reinterpret_cast<const u32x4_t*>(q_base + (int64_t)qr * a.qs[1] + dc);
+            u32x4_t gv = *reinterpret_cast<const u32x4_t*>(g_base + (int64_t)qr * a.os[1] + dc);
+            if (q_row >= a.sq || d0 >= a.d) {
+                qv = u32x4_t{0u, 0u, 0u, 0u};
+                gv = u32x4_t{0u, 0u, 0u, 0u};
+            }
+            qf[t] = __builtin_bit_cast(frag_t, qv);
+            gf[t] = __builtin_bit_cast(frag_t, gv);
+        }
+        if (q_row < a.sq) {
+            lse2 = a.lse[(int64_t)bh * a.sq + q_row] * kLog2e;
+            delta = a.delta[(int64_t)bh * a.sq + q_row];
+        }
+    }
+
+    f32x16_t dq_acc[DV];
+#pragma unroll
+    for (int x = 0; x < DV; ++x)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dq_acc[x][r] = 0.f;
+
+    int j_lo, j_hi;
+    key_range(a, q0, min(q0 + kBM, a.sq), j_lo, j_hi);
+    const int t_lo = j_lo / kBN;
+    const int t_hi = (j_hi + kBN - 1) / kBN;
+    const int n_tiles = t_hi - t_lo;
+
+    const int wq_last = min(wq0 + 31, a.sq - 1);
+    const float c_log2 = a.scale_log2;
+    uint64_t drop_row_base = 0;
+    if constexpr (kDropout)
+        drop_row_base = ((uint64_t)bh * a.sq + (uint64_t)q_row) * (uint64_t)a.sk;
+    const float* bias_row = nullptr;
+    if constexpr (kBias)
+        bias_row = a.bias + b * a.bs[0] + h * a.bs[1] + (int64_t)min(q_row, a.sq - 1) * a.bs[2];
+
+    // per-lane LDS offsets (elements) that do not change from tile to tile
+    const int row_off = pi_row(i_loc) * kPitch + 8 * g;
+    const int tr_off = (8 * g + ((lane & 15) >> 2)) * kPitch + ((lane >> 4) & 1) * 16 + 4 * (lane & 3);
+
+    auto tile_active = [&](int t) __attribute__((always_inline)) {
+        if (t < t_lo || t >= t_hi || wq0 >= a.sq) return false;
+        const int j0 = t * kBN;
+        if (a.causal && j0 > wq_last) return false;
+        if (a.window > 0 && wq0 - (j0 + kBN - 1) >= a.window) return false;
+        return true;
+    };
+    auto tile_needs_mask = [&](int t) __attribute__((always_inline)) {
+        const int j0 = t * kBN;
+        return (j0 + kBN > a.sk) || (a.causal && j0 + kBN - 1 > wq0) ||
+               (a.window > 0 && wq_last - j0 >= a.window);
+    };
+
+    // The tile is processed as two halves of 32 keys whose stages are staggered, so that the matrix
+    // instructions of one half always have independent vector work of the other half around them
+    // (a wavefront overlaps the two only when they are interleaved in its instruction stream).
+
+    // S^T half = K_half Q^T
+    auto half_s = [&](const T* kt, int kb, f32x16_t& s) __attribute__((always_inline)) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[r] = 0.f;
+#pragma unroll
+        for (int x = 0; x < DK; ++x)
+            s = Mma<T>::mma32(lds_frag<T>(kt + kb * 32 * kPitch + row_off + 16 * x), qf[x], s);
+    };
+    // dP^T half = V_half dO^T
+    auto half_dp = [&](const T* vt, int kb, f32x16_t& dp) __attribute__((always_inline)) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dp[r] = 0.f;
+#pragma unroll
+        for (int x = 0; x < DK; ++x)
+            dp = Mma<T>::mma32(lds_frag<T>(vt + kb * 32 * kPitch + row_off + 16 * x), gf[x], dp);
+    };
+    // dQ^T += K_half^T dS^T half
+    auto half_dq = [&](const T* kt, int kb, const uint32_t (&dw)[8]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+            u32x4_t dq4 = {dw[4 * s2], dw[4 * s2 + 1], dw[4 * s2 + 2], dw[4 * s2 + 3]};
+            const frag_t df = __builtin_bit_cast(frag_t, dq4);
+#pragma unroll
+            for (int x = 0; x < DV; ++x)
+                dq_acc[x] = Mma<T>::mma32(
+                    lds_frag_tr<T>(kt + (32 * kb + 16 * s2) * kPitch + tr_off + 32 * x, kPitch), df,
+                    dq_acc[x]);
+        }
+    };
+    // scores -> probabilities, in place
+    // mask_tag: 0 = every key visible, 1 = upper bound only (causal / key tail), 2 = both bounds
+    auto half_exp = [&](f32x16_t& s, int t, int kb, auto mask_tag) __attribute__((always_inline)) {
+        constexpr int kMask = decltype(mask_tag)::value;
+        const int j0 = t * kBN + kb * 32;
+        // register r is key j0 + 8 g + c with c = acc_row(r, 0); visible iff c_lo <= c <= c_hi
+        int c_lo = 0, c_hi = 0;
+        if constexpr (kMask != 0) {
+            const int k_max = a.causal ? min(a.sk - 1, q_row) : a.sk - 1;
+            c_hi = k_max - j0 - 8 * g;
+            if constexpr (kMask == 2) c_lo = q_row - a.window + 1 - j0 - 8 * g;
+        }
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) {
+            float bv[4] = {0.f, 0.f, 0.f, 0.f};
+            if constexpr (kBias) {
+                const int key0 = j0 + acc_row(4 * r4, g);
+                if (a.bias_vec4 && key0 + 3 < a.sk) {
+                    const f32x4_t t4 = *reinterpret_cast<const f32x4_t*>(bias_row + key0);
+                    bv[0] = t4.x, bv[1] = t4.y, bv[2] = t4.z, bv[3] = t4.w;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (key0 + e < a.sk) bv[e] = bias_row[(int64_t)(key0 + e) * a.bs[3]];
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                float x = __builtin_fmaf(s[4 * r4 + e], c_log2, -lse2);
+                if constexpr (kBias) x = __builtin_fmaf(bv[e], kLog2e, x);
+                float p = fast_exp2(x);
+                if constexpr (kMask != 0) {
+                    const int c = acc_row(4 * r4, 0) + e;
+                    if constexpr (kMask == 2) {
+                        if (c > c_hi || c < c_lo) p = 0.f;
+                    } else {
+                        if (c > c_hi) p = 0.f;
+                    }
+                }
+                s[4 * r4 + e] = p;
+            }
+        }
+    };
+    // dS^T half = P^T (dP^T - delta), packed to T
+    auto half_ds = [&](const f32x16_t& p, const f32x16_t& dp, int t, int kb, uint32_t (&dw)[8])
+                       __attribute__((always_inline)) {
+        const int j0 = t * kBN + kb * 32;
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) {
+            uint32_t bits = 0xFu;
+            if constexpr (kDropout) {
+                const int key0 = j0 + acc_row(4 * r4, g);
+                bits = 0;
+                if (q_row < a.sq && key0 < a.sk) {
+                    const uint64_t e0 = drop_row_base + (uint64_t)key0;
+                    if (a.dropout_fast) {
+                        bits = dropout_keep4(a.rng, e0 >> 2);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e)
+                            if (key0 + e < a.sk)
+                                bits |= (dropout_keep1(a.rng, e0 + e) ? 1u : 0u) << e;
+                    }
+                }
+            }
+            float dv[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                float d = dp[4 * r4 + e];
+                if constexpr (kDropout) d = ((bits >> e) & 1u) ? d * a.rng.inv_keep : 0.f;
+                dv[e] = p[4 * r4 + e] * (d - delta);
+            }
+            dw[2 * r4] = pack2<T>(dv[0], dv[1]);
+            dw[2 * r4 + 1] = pack2<T>(dv[2], dv[3]);
+        }
+    };
+    auto tile_body = [&](const T* kt, const T* vt, int t, auto mask_tag) __attribute__((always_inline)) {
+        f32x16_t s0, s1, p0, p1;
+        uint32_t dw0[8], dw1[8];
+        half_s(kt, 0, s0);
+        half_dp(vt, 0, p0);
+        half_exp(s0, t, 0, mask_tag);
+        half_s(kt, 1, s1);
+        half_ds(s0, p0, t, 0, dw0);
+        half_dp(vt, 1, p1);
+        half_exp(s1, t, 1, mask_tag);
+        half_dq(kt, 0, dw0);
+        half_ds(s1, p1, t, 1, dw1);
+        half_dq(kt, 1, dw1);
+    };
+
+    // ---- prologue: tile 0 into LDS ----
+    Stage ks, vs;
+    if (n_tiles > 0) {
+        ks.load(k_base, a.ks[1], t_lo * kBN, a.sk, a.d);
+        vs.load(v_base, a.vs[1], t_lo * kBN, a.sk, a.d);
+        ks.fix(t_lo * kBN, a.sk, a.d);
+        vs.fix(t_lo * kBN, a.sk, a.d);
+        ks.store(k_lds);
+        vs.store(v_lds);
+    }
+    __syncthreads();
+
+    // Iteration r: request tile r+1, process tile r, write tile r+1 into the other ring slot.
+    // kFast iterations hold tiles that every wavefront of the workgroup sees in full, so their body
+    // is one straight block; the others test activity and masks per wavefront.
+    auto iteration = [&](int r, auto fast_tag) __attribute__((always_inline)) {
+        constexpr bool kFast = decltype(fast_tag)::value;
+        const int t = t_lo + r;
+        const bool have_next = r + 1 < n_tiles;
+        if (have_next) {
+            ks.load(k_base, a.ks[1], (t + 1) * kBN, a.sk, a.d);
+            vs.load(v_base, a.vs[1], (t + 1) * kBN, a.sk, a.d);
+        }
+        const T* kt = k_lds + (r % kKRing) * kTileElems;
+        const T* vt = v_lds + (r % kVRing) * kTileElems;
+        if constexpr (kFast) {
+            tile_body(kt, vt, t, std::integral_constant<int, 0>{});
+        } else if (tile_active(t)) {
+            if (!tile_needs_mask(t))
+                tile_body(kt, vt, t, std::integral_constant<int, 0>{});
+            else if (a.window > 0)
+                tile_body(kt, vt, t, std::integral_constant<int, 2>{});
+            else
+                tile_body(kt, vt, t, std::integral_constant<int, 1>{});
+        }
+        if (have_next) {
+            ks.fix((t + 1) * kBN, a.sk, a.d);
+            vs.fix((t + 1) * kBN, a.sk, a.d);
+            ks.store(k_lds + ((r + 1) % kKRing) * kTileElems);
+            vs.store(v_lds + ((r + 1) % kVRing) * kTileElems);
+        }
+        __syncthreads();
+    };
+    // leading tiles that need neither mask nor activity test for any of the 128 queries
+    int n_fast = 0;
+    if (a.window <= 0 && q0 + kBM <= a.sq) {
+        n_fast = a.sk / kBN;
+        if (a.causal) n_fast = min(n_fast, (q0 + 1) / kBN);
+        n_fast = min(n_fast, n_tiles);
+    }
+    int r = 0;
+    for (; r < n_fast; ++r) iteration(r, std::true_type{});
+    for (; r < n_tiles; ++r) iteration(r, std::false_type{});
+
+    // ---- epilogue: dQ = scale * dQ^T^T ----
+    if (q_row < a.sq) {
+        T* dq_row =
+            reinterpret_cast<T*>(a.dq) + b * a.dqs[0] + (int64_t)q_row * a.dqs[1] + h * a.dqs[2];
+#pragma unroll
+        for (int x = 0; x < DV; ++x)
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                const int d0 = x * 32 + 8 * r4 + 4 * g;
+                if (d0 < a.d) {
+                    u32x2_t w;
+                    w.x = pack2<T>(dq_acc[x][4 * r4 + 0] * a.scale, dq_acc[x][4 * r4 + 1] * a.scale);
+                    w.y = pack2<T>(dq_acc[x][4 * r4 + 2] * a.scale, dq_acc[x][4 * r4 + 3] * a.scale);
+                    *reinterpret_cast<u32x2_t*>(dq_row + d0) = w;
+                }
+            }
+    }
+}
+
+template <typename T, int DPAD, bool kBias, bool kDropout>
+int launch(const AttnArgs& a, hipStream_t st) {
+    typedef TileStage<T, DPAD, kBN, kThreads> Stage;
+    const size_t smem = (size_t)(kKRing + kVRing) * kBN * Stage::kPitch * sizeof(T);
+    const int n_qt = (a.sq + kBM - 1) / kBM;
+    const int64_t blocks = (int64_t)n_qt * a.batch * a.heads;
+    if (blocks <= 0 || blocks > 0x7FFFFFFF) return SLAPO_ERR_SHAPE;
+    auto kern = attn_bwd_dq_kernel<T, DPAD, kBias, kDropout>;
+    if (smem > 48 * 1024) {
+        static bool raised = false;  // per instantiation
+        if (!raised) {
+            if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)smem) != hipSuccess)
+                return SLAPO_ERR_LAUNCH;
+            raised = true;
+        }
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kThreads), smem, st, a);
+    return check_launch();
+}
+
+template <typename T, int DPAD>
+int dispatch_flags(const AttnArgs& a, hipStream_t st) {
+    if (a.has_bias) {
+        if (a.dropout) return launch<T, DPAD, true, true>(a, st);
+        return launch<T, DPAD, true, false>(a, st);
+    }
+    if (a.dropout) return launch<T, DPAD, false, true>(a, st);
+    return launch<T, DPAD, false, false>(a, st);
+}
+
+template <typename T>
+int dispatch(const AttnArgs& a, hipStream_t st) {
+    if (a.d <= 64) return dispatch_flags<T, 64>(a, st);
+    if (a.d <= 96) return dispatch_flags<T, 96>(a, st);
+    if (a.d <= 128) return dispatch_flags<T, 128>(a, st);
+    return SLAPO_ERR_SHAPE;
+}
+
+}  // namespace bwd_dq
+}  // namespace slapo

@@ -1,4 +1,4 @@
-// Flash-attention backward for gfx950, fp16 / bf16 inputs, fp32 accumulation.
+// Flash-attention backward, dK / dV half, for gfx950 (fp16 / bf16 inputs, fp32 accumulation).
 //
 // One workgroup (4 wavefronts) owns 128 consecutive keys of one (batch, head); wavefront w owns
 // 32 of them and keeps their K and V fragments in registers for the whole kernel, together with
@@ -14,19 +14,11 @@
 //                                    (the row permutation makes them ordered k-slots), A = dO^T /
 //                                    Q^T read from the same row-major LDS tiles with the
 //                                    transposing LDS read.
-//   dQ += dS K                       dS goes through LDS once ([key][query], double buffered);
-//                                    after the barrier each wavefront computes 16 head-dim
-//                                    columns of dQ over ALL 128 keys of the workgroup with
-//                                    16x16x32 MFMAs (A = dS via the transposing read, B = K^T
-//                                    fragments resident in registers) and adds the tile into the
-//                                    fp32 dQ accumulator with hardware float atomics: one atomic
-//                                    tile per workgroup and query tile instead of one per
-//                                    wavefront.
-// One barrier per query tile.  Reference semantics: autograd of slapo/op/attention.py:163-181.
+// dQ is produced by the sibling kernel that owns query rows, so nothing here is shared between
+// workgroups.  One barrier per query tile.
+// Reference semantics: autograd of slapo/op/attention.py:163-181.
 #pragma once
 #include <cstdio>
-#include <hip/amd_detail/amd_hip_unsafe_atomics.h>
-
 #include <type_traits>
 
 #include "attn_common.h"
@@ -38,21 +30,15 @@ constexpr int kBwdWaves = 4;
 constexpr int kBwdThreads = kBwdWaves * 64;
 constexpr int kBwdBN = kBwdWaves * 32;  // keys per workgroup
 constexpr int kBwdBM = 32;              // queries per tile
-constexpr int kDsPitch = kBwdBM + 8;    // dS tile [key][query] row pitch (elements)
 
 template <typename T, int DPAD>
 struct BwdSmem {
     typedef TileStage<T, DPAD, kBwdBM, kBwdThreads> QStage;
     static constexpr int kPitch = QStage::kPitch;
     static constexpr int kQTile = kBwdBM * kPitch;            // elements
-    static constexpr int kDsTile = kBwdBN * kDsPitch;         // elements
-    static constexpr int kKStage = kBwdBN * kPitch;           // elements (start-up only)
     static constexpr size_t kQBytes = 2 * kQTile * sizeof(T);   // double buffered
-    static constexpr size_t kDsBytes = 2 * kDsTile * sizeof(T);
     static constexpr size_t kStatBytes = 2 * 2 * kBwdBM * sizeof(float);
-    static constexpr size_t kLoopBytes = 2 * kQBytes + kDsBytes + kStatBytes;
-    static constexpr size_t kStageBytes = kKStage * sizeof(T);
-    static constexpr size_t kBytes = kLoopBytes > kStageBytes ? kLoopBytes : kStageBytes;
+    static constexpr size_t kBytes = 2 * kQBytes + kStatBytes;
 };
 
 template <typename T, int DPAD, bool kBias, bool kDropout>
@@ -64,15 +50,11 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
     constexpr int kPitch = SM::kPitch;
     constexpr int DK = DPAD / 16;          // k-steps over head dim
     constexpr int DV = DPAD / 32;          // 32-row blocks of dK^T / dV^T
-    constexpr int NBLK = DPAD / 16;        // 16-column blocks of dQ
-    constexpr int NDB = (NBLK + kBwdWaves - 1) / kBwdWaves;  // dQ blocks per wavefront
 
     extern __shared__ __align__(16) unsigned char smem_raw[];
     T* q_lds = reinterpret_cast<T*>(smem_raw);
     T* g_lds = reinterpret_cast<T*>(smem_raw + SM::kQBytes);
-    T* ds_lds = reinterpret_cast<T*>(smem_raw + 2 * SM::kQBytes);
-    float* stat_lds = reinterpret_cast<float*>(smem_raw + 2 * SM::kQBytes + SM::kDsBytes);
-    T* kstage = reinterpret_cast<T*>(smem_raw);
+    float* stat_lds = reinterpret_cast<float*>(smem_raw + 2 * SM::kQBytes);
 
     const int n_bh = a.batch * a.heads;
     const int bh = blockIdx.x % n_bh;
@@ -82,7 +64,7 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
     const int k0 = kt * kBwdBN;
 
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wavefront-uniform
     const int g = lane >> 5;
     const int c_loc = lane & 31;
 #ifdef EXP_TIMING
@@ -106,7 +88,6 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
     const T* g_base = reinterpret_cast<const T*>(a.dout) + b * a.os[0] + h * a.os[2];
     const float* lse_base = a.lse + (int64_t)bh * a.sq;
     const float* delta_base = a.delta + (int64_t)bh * a.sq;
-    float* dq_base = reinterpret_cast<float*>(a.dq) + (int64_t)bh * a.sq * a.d;
 
     // ---- resident fragments ----
     frag_t kf[DK], vf[DK];
@@ -121,33 +102,6 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
         kf[t] = __builtin_bit_cast(frag_t, kv);
         vf[t] = __builtin_bit_cast(frag_t, vv);
     }
-    // K^T fragments for dQ = dS K: B operand of the 16x16x32 MFMA, column d, k-slots = keys.
-    frag_t ktf[NDB][kBwdWaves];
-    {
-        TileStage<T, DPAD, kBwdBN, kBwdThreads> kst;
-        kst.load(k_base, a.ks[1], k0, a.sk, a.d);
-        kst.fix(k0, a.sk, a.d);
-        kst.store(kstage);
-        __syncthreads();
-        const int beta = lane >> 4;
-#pragma unroll
-        for (int nb = 0; nb < NDB; ++nb) {
-            const int blk = wave + nb * kBwdWaves;
-#pragma unroll
-            for (int st = 0; st < kBwdWaves; ++st) {
-                if (blk < NBLK) {
-                    const T* src = kstage + (32 * st + 8 * beta + ((lane & 15) >> 2)) * kPitch +
-                                   16 * blk + 4 * (lane & 3);
-                    ktf[nb][st] = lds_frag_tr<T>(src, kPitch);
-                } else {
-                    u32x4_t z = {0u, 0u, 0u, 0u};
-                    ktf[nb][st] = __builtin_bit_cast(frag_t, z);
-                }
-            }
-        }
-        __syncthreads();
-    }
-
     f32x16_t dk_acc[DV], dv_acc[DV];
 #pragma unroll
     for (int x = 0; x < DV; ++x)
@@ -171,8 +125,6 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
     // per-lane LDS offsets (elements) that do not change from tile to tile
     const int a_off = pi_row(c_loc) * kPitch + 8 * g;
     const int t_off = (8 * g + ((lane & 15) >> 2)) * kPitch + ((lane >> 4) & 1) * 16 + 4 * (lane & 3);
-    const int ds_w_off = (wave * 32 + c_loc) * kDsPitch;
-    const int ds_r_off = (8 * (lane >> 4) + ((lane & 15) >> 2)) * kDsPitch + 4 * (lane & 3);
 
     QStage qst, gst;
     // lse / delta of a query tile: threads 0..31 fetch lse, threads 32..63 delta.  The load is
@@ -213,60 +165,13 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
         return true;
     };
 
-    // dQ tile = dS K over all active key slabs of the workgroup, for the query tile at i0 whose
-    // dS^T sits in `dst`; added to the fp32 accumulator with hardware atomics.
-    auto dq_phase = [&](const T* dst, int i0) __attribute__((always_inline)) {
-        const int beta = lane >> 4;
-        const int n16 = lane & 15;
-#pragma unroll
-        for (int nb = 0; nb < NDB; ++nb) {
-            const int blk = wave + nb * kBwdWaves;
-            if (blk >= NBLK) continue;
-            f32x4_t acc[2];
-#pragma unroll
-            for (int qb = 0; qb < 2; ++qb) acc[qb] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-            bool any = false;
-#pragma unroll
-            for (int st = 0; st < kBwdWaves; ++st) {
-                if (!slab_active(st, i0)) continue;
-                any = true;
-                const T* src = dst + 32 * st * kDsPitch + ds_r_off;
-#pragma unroll
-                for (int qb = 0; qb < 2; ++qb)
-                    acc[qb] = Mma<T>::mma16(lds_frag_tr<T>(src + 16 * qb, kDsPitch), ktf[nb][st],
-                                            acc[qb]);
-            }
-            if (!any) continue;
-            const int dcol = 16 * blk + n16;
-            float* dq_col = dq_base + (int64_t)(i0 + 4 * beta) * a.d + dcol;
-            if (i0 + kBwdBM <= a.sq && dcol < a.d) {
-#pragma unroll
-                for (int qb = 0; qb < 2; ++qb)
-#pragma unroll
-                    for (int r = 0; r < 4; ++r)
-                        unsafeAtomicAdd(dq_col + (int64_t)(16 * qb + r) * a.d, acc[qb][r]);
-            } else if (dcol < a.d) {
-#pragma unroll
-                for (int qb = 0; qb < 2; ++qb)
-#pragma unroll
-                    for (int r = 0; r < 4; ++r)
-                        if (i0 + 16 * qb + 4 * beta + r < a.sq)
-                            unsafeAtomicAdd(dq_col + (int64_t)(16 * qb + r) * a.d, acc[qb][r]);
-            }
-        }
-    };
-
     TSTAMP();
-    // Iteration t: request tile t+1, run the dQ phase of tile t-1 (its dS^T was completed before the
-    // last barrier), then the S / dP / dV / dK work of tile t, then write tile t+1 to LDS.
-    // One extra trip drains the dQ phase of the last tile.
-    for (int t = t_lo; t <= t_hi; ++t) {
+    // Iteration t: request tile t+1, do the S / dP / dV / dK work of tile t, write tile t+1 to LDS.
+    for (int t = t_lo; t < t_hi; ++t) {
         TSTAMP();
-        const bool compute = t < t_hi;
         const int buf = (t - t_lo) & 1;
         const T* qt = q_lds + buf * SM::kQTile;
         const T* gt = g_lds + buf * SM::kQTile;
-        T* dst = ds_lds + buf * SM::kDsTile;
         const float* lse_t = stat_lds + buf * 64;
         const float* delta_t = lse_t + 32;
         const int i0 = t * kBwdBM;
@@ -276,10 +181,8 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
             gst.load(g_base, a.os[1], i0 + kBwdBM, a.sq, a.d);
             load_stats(i0 + kBwdBM);
         }
-        if (t > t_lo) dq_phase(ds_lds + (buf ^ 1) * SM::kDsTile, i0 - kBwdBM);
-
         const int i_last = min(i0 + kBwdBM, a.sq) - 1;
-        const bool active = compute && slab_active(wave, i0);
+        const bool active = slab_active(wave, i0);
 
         auto tile_body = [&](auto mask_tag) __attribute__((always_inline)) {
             constexpr bool kMask = decltype(mask_tag)::value;
@@ -343,9 +246,6 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
                 pw[2 * r4 + 1] = pack2<T>(pv[2], pv[3]);
                 dw[2 * r4] = pack2<T>(dv[0], dv[1]);
                 dw[2 * r4 + 1] = pack2<T>(dv[2], dv[3]);
-                // dS^T slab for the dQ pass: row = key (local), columns = 4 consecutive queries
-                u32x2_t w2 = {dw[2 * r4], dw[2 * r4 + 1]};
-                *reinterpret_cast<u32x2_t*>(dst + ds_w_off + qoff) = w2;
             }
             // ---- dV^T += dO^T P,  dK^T += Q^T dS ----
 #pragma unroll
@@ -383,7 +283,7 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
             store_stats(buf ^ 1, i0 + kBwdBM);
         }
         TSTAMP();
-        if (compute) __syncthreads();
+        __syncthreads();
         TSTAMP();
     }
 

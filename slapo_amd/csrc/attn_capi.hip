@@ -1,6 +1,6 @@
 // C-ABI entry points of the attention path: argument validation, kernel selection (MFMA kernels
 // for fp16 / bf16, FMA kernels for fp32) and the small helper kernels around the backward
-// (delta = rowsum(dO * O), dQ accumulator clear and fp32 -> T conversion).
+// (delta = rowsum(dO * O)).
 #include "attn_common.h"
 
 namespace slapo {
@@ -8,6 +8,8 @@ int attn_fwd_mfma_f16(const AttnArgs& a, hipStream_t st);
 int attn_fwd_mfma_bf16(const AttnArgs& a, hipStream_t st);
 int attn_bwd_mfma_f16(const AttnArgs& a, hipStream_t st);
 int attn_bwd_mfma_bf16(const AttnArgs& a, hipStream_t st);
+int attn_bwd_dq_mfma_f16(const AttnArgs& a, hipStream_t st);
+int attn_bwd_dq_mfma_bf16(const AttnArgs& a, hipStream_t st);
 int attn_fwd_f32(const AttnArgs& a, hipStream_t st);
 int attn_bwd_f32(const AttnArgs& a, hipStream_t st);
 }  // namespace slapo
@@ -17,10 +19,8 @@ using namespace slapo;
 namespace {
 
 // delta[bh, i] = sum_d dO[b,i,h,d] * O[b,i,h,d]; eight lanes share a row, 16 bytes per lane.
-// When zero_acc is given, the same lanes also clear row (bh, i) of the fp32 dQ accumulator, so the
-// backward needs one preparation launch instead of two.
 template <typename T>
-__global__ __launch_bounds__(256) void attn_delta_kernel(const AttnArgs a, float* zero_acc) {
+__global__ __launch_bounds__(256) void attn_delta_kernel(const AttnArgs a) {
     constexpr int V = Elem<T>::kPerVec;
     const int64_t row = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 3;
     const int sub = threadIdx.x & 7;
@@ -42,11 +42,6 @@ __global__ __launch_bounds__(256) void attn_delta_kernel(const AttnArgs a, float
                 acc = __builtin_fmaf(Elem<T>::to_f32(po.v[e]), Elem<T>::to_f32(pg.v[e]), acc);
         }
     }
-    if (zero_acc && row < n_rows) {
-        float* z = zero_acc + row * a.d;
-        for (int c = sub * 4; c < a.d; c += 32)
-            *reinterpret_cast<f32x4_t*>(z + c) = f32x4_t{0.f, 0.f, 0.f, 0.f};
-    }
     acc += __shfl_xor(acc, 1, 64);
     acc += __shfl_xor(acc, 2, 64);
     acc += __shfl_xor(acc, 4, 64);
@@ -67,27 +62,6 @@ __global__ __launch_bounds__(256) void attn_delta_scalar_kernel(const AttnArgs a
     float acc = 0.f;
     for (int e = 0; e < a.d; ++e) acc = __builtin_fmaf(o[e], g[e], acc);
     a.delta[row] = acc;
-}
-
-// dq[b,i,h,:] = T(scale * dq_acc[bh,i,:]);  8 lanes per row, 4 floats per lane per trip.
-template <typename T>
-__global__ __launch_bounds__(256) void dq_convert_kernel(const AttnArgs a, const float* acc) {
-    const int64_t row = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 3;
-    const int sub = threadIdx.x & 7;
-    const int64_t n_rows = (int64_t)a.batch * a.heads * a.sq;
-    if (row >= n_rows) return;
-    const int i = (int)(row % a.sq);
-    const int bh = (int)(row / a.sq);
-    const int b = bh / a.heads, h = bh % a.heads;
-    T* out = reinterpret_cast<T*>(a.dq) + b * a.dqs[0] + (int64_t)i * a.dqs[1] + h * a.dqs[2];
-    const float* src = acc + row * a.d;
-    for (int c = sub * 4; c < a.d; c += 32) {
-        const f32x4_t v = *reinterpret_cast<const f32x4_t*>(src + c);
-        u32x2_t w;
-        w.x = pack2<T>(v.x * a.scale, v.y * a.scale);
-        w.y = pack2<T>(v.z * a.scale, v.w * a.scale);
-        *reinterpret_cast<u32x2_t*>(out + c) = w;
-    }
 }
 
 bool strides_ok(const int64_t s[3], int mult) {
@@ -191,9 +165,7 @@ extern "C" size_t slapo_amd_attn_bwd_workspace_bytes(const slapo_attn_params* pr
     if (!prm || prm->batch <= 0 || prm->heads <= 0 || prm->seqlen_q <= 0 || prm->head_dim <= 0)
         return 0;
     const size_t rows = (size_t)prm->batch * prm->heads * prm->seqlen_q;
-    size_t bytes = rows * sizeof(float);  // delta
-    if (prm->dtype != SLAPO_F32) bytes += rows * (size_t)prm->head_dim * sizeof(float);  // dQ acc
-    return bytes;
+    return rows * sizeof(float);  // delta
 }
 
 extern "C" int slapo_amd_attn_bwd_stages(const slapo_attn_params* prm, const void* q,
@@ -226,9 +198,8 @@ extern "C" int slapo_amd_attn_bwd_stages(const slapo_attn_params* prm, const voi
 
     const int64_t rows = (int64_t)a.batch * a.heads * a.sq;
     const bool is_f32 = prm->dtype == SLAPO_F32;
-    // workspace: [dQ accumulator (16-bit types only)] [delta]
-    float* dq_acc = reinterpret_cast<float*>(workspace);
-    a.delta = is_f32 ? dq_acc : dq_acc + rows * a.d;
+    a.delta = reinterpret_cast<float*>(workspace);
+    a.dq = dq;
 
     if (is_f32) {
         if (stages & SLAPO_BWD_PREPARE) {
@@ -236,8 +207,7 @@ extern "C" int slapo_amd_attn_bwd_stages(const slapo_attn_params* prm, const voi
                                 strides_ok(prm->o_strides, 4);
             if (vec_ok) {
                 const unsigned blocks = (unsigned)((rows * 8 + 255) / 256);
-                hipLaunchKernelGGL((attn_delta_kernel<float>), dim3(blocks), dim3(256), 0, st, a,
-                                   (float*)nullptr);
+                hipLaunchKernelGGL((attn_delta_kernel<float>), dim3(blocks), dim3(256), 0, st, a);
             } else {
                 const unsigned blocks = (unsigned)((rows + 255) / 256);
                 hipLaunchKernelGGL(attn_delta_scalar_kernel, dim3(blocks), dim3(256), 0, st, a);
@@ -245,10 +215,7 @@ extern "C" int slapo_amd_attn_bwd_stages(const slapo_attn_params* prm, const voi
             rc = check_launch();
             if (rc != SLAPO_OK) return rc;
         }
-        if (stages & SLAPO_BWD_MAIN) {
-            a.dq = dq;
-            rc = attn_bwd_f32(a, st);
-        }
+        if (stages & SLAPO_BWD_DKDV) rc = attn_bwd_f32(a, st);
         return rc;
     }
 
@@ -256,20 +223,17 @@ extern "C" int slapo_amd_attn_bwd_stages(const slapo_attn_params* prm, const voi
     if (!strides_ok(dq_strides, 8) || !strides_ok(dk_strides, 8) || !strides_ok(dv_strides, 8))
         return SLAPO_ERR_ALIGN;
 
-    const unsigned row_blocks = (unsigned)((rows * 8 + 255) / 256);
     if (stages & SLAPO_BWD_PREPARE) {
-        // head_dim % 8 == 0, so each accumulator row is a whole number of 16-byte stores
+        const unsigned row_blocks = (unsigned)((rows * 8 + 255) / 256);
         if (prm->dtype == SLAPO_F16)
-            hipLaunchKernelGGL((attn_delta_kernel<f16_t>), dim3(row_blocks), dim3(256), 0, st, a,
-                               dq_acc);
+            hipLaunchKernelGGL((attn_delta_kernel<f16_t>), dim3(row_blocks), dim3(256), 0, st, a);
         else
-            hipLaunchKernelGGL((attn_delta_kernel<bf16_t>), dim3(row_blocks), dim3(256), 0, st, a,
-                               dq_acc);
+            hipLaunchKernelGGL((attn_delta_kernel<bf16_t>), dim3(row_blocks), dim3(256), 0, st, a);
         rc = check_launch();
         if (rc != SLAPO_OK) return rc;
     }
-    if (stages & SLAPO_BWD_MAIN) {
-        a.dq = dq_acc;
+    // dK / dV (workgroups own keys), then dQ (workgroups own queries); both read delta.
+    if (stages & SLAPO_BWD_DKDV) {
 #ifdef EXP_TIMING
         if (!g_timing_buf) { hipMalloc(&g_timing_buf, 1 << 16); hipMemset(g_timing_buf, 0, 1 << 16); }
         a.o = g_timing_buf;
@@ -277,16 +241,8 @@ extern "C" int slapo_amd_attn_bwd_stages(const slapo_attn_params* prm, const voi
         rc = prm->dtype == SLAPO_F16 ? attn_bwd_mfma_f16(a, st) : attn_bwd_mfma_bf16(a, st);
         if (rc != SLAPO_OK) return rc;
     }
-    if (stages & SLAPO_BWD_FINISH) {
-        a.dq = dq;
-        if (prm->dtype == SLAPO_F16)
-            hipLaunchKernelGGL((dq_convert_kernel<f16_t>), dim3(row_blocks), dim3(256), 0, st, a,
-                               dq_acc);
-        else
-            hipLaunchKernelGGL((dq_convert_kernel<bf16_t>), dim3(row_blocks), dim3(256), 0, st, a,
-                               dq_acc);
-        rc = check_launch();
-    }
+    if (stages & SLAPO_BWD_DQ)
+        rc = prm->dtype == SLAPO_F16 ? attn_bwd_dq_mfma_f16(a, st) : attn_bwd_dq_mfma_bf16(a, st);
     return rc;
 }
 
