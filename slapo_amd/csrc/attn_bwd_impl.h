@@ -2,8 +2,8 @@
 //
 // One workgroup (4 wavefronts) owns 128 consecutive keys of one (batch, head); wavefront w owns
 // 32 of them and keeps their K and V fragments in registers for the whole kernel, together with
-// its dK^T and dV^T accumulators.  Query tiles of 32 rows (Q, dO, lse, delta) stream through LDS,
-// double buffered and staged through registers.  Per query tile and wavefront (lane l,
+// its dK^T and dV^T accumulators.  Query tiles of 64 rows (Q, dO, lse, delta) stream through LDS,
+// double buffered and staged through registers.  Per 32-query half tile and wavefront (lane l,
 // g = l / 32):
 //   S  = Q K_w^T, dP = dO V_w^T      A = Q / dO rows from LDS (row-permuted 128-bit reads),
 //                                    B = the resident K_w / V_w fragments.  Lane l holds one KEY
@@ -14,8 +14,10 @@
 //                                    (the row permutation makes them ordered k-slots), A = dO^T /
 //                                    Q^T read from the same row-major LDS tiles with the
 //                                    transposing LDS read.
-// dQ is produced by the sibling kernel that owns query rows, so nothing here is shared between
-// workgroups.  One barrier per query tile.
+// The two halves of a tile are staggered so that the matrix instructions of one half have vector
+// work of the other half around them (a wavefront overlaps the two only when they are interleaved
+// in its instruction stream).  dQ is produced by the sibling kernel that owns query rows, so
+// nothing here is shared between workgroups.  One barrier per query tile.
 // Reference semantics: autograd of slapo/op/attention.py:163-181.
 #pragma once
 #include <cstdio>
@@ -29,7 +31,7 @@ namespace bwd {
 constexpr int kBwdWaves = 4;
 constexpr int kBwdThreads = kBwdWaves * 64;
 constexpr int kBwdBN = kBwdWaves * 32;  // keys per workgroup
-constexpr int kBwdBM = 32;              // queries per tile
+constexpr int kBwdBM = 64;              // queries per tile
 
 template <typename T, int DPAD>
 struct BwdSmem {
@@ -37,7 +39,7 @@ struct BwdSmem {
     static constexpr int kPitch = QStage::kPitch;
     static constexpr int kQTile = kBwdBM * kPitch;            // elements
     static constexpr size_t kQBytes = 2 * kQTile * sizeof(T);   // double buffered
-    static constexpr size_t kStatBytes = 2 * 2 * kBwdBM * sizeof(float);
+    static constexpr size_t kStatBytes = 2 * 2 * kBwdBM * sizeof(float);  // lse, delta; x2 buffers
     static constexpr size_t kBytes = 2 * kQBytes + kStatBytes;
 };
 
@@ -127,19 +129,21 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
     const int t_off = (8 * g + ((lane & 15) >> 2)) * kPitch + ((lane >> 4) & 1) * 16 + 4 * (lane & 3);
 
     QStage qst, gst;
-    // lse / delta of a query tile: threads 0..31 fetch lse, threads 32..63 delta.  The load is
+    // lse / delta of a query tile: threads 0..63 fetch lse, threads 64..127 delta.  The load is
     // unconditional (row clamped) and its result is not touched until the tile is written to LDS.
     float stat_reg = 0.f;
-    const float* stat_src = (threadIdx.x < 32) ? lse_base : delta_base;
+    const float* stat_src = (threadIdx.x < kBwdBM) ? lse_base : delta_base;
     auto load_stats = [&](int i0) __attribute__((always_inline)) {
-        if (threadIdx.x < 64) stat_reg = stat_src[min(i0 + (int)(threadIdx.x & 31), a.sq - 1)];
+        if (threadIdx.x < 2 * kBwdBM)
+            stat_reg = stat_src[min(i0 + (int)(threadIdx.x & (kBwdBM - 1)), a.sq - 1)];
     };
     auto store_stats = [&](int buf, int i0) __attribute__((always_inline)) {
-        if (threadIdx.x < 64) {
-            const bool ok = i0 + (int)(threadIdx.x & 31) < a.sq;
+        if (threadIdx.x < 2 * kBwdBM) {
+            const bool ok = i0 + (int)(threadIdx.x & (kBwdBM - 1)) < a.sq;
             // lse in log2 units, +inf for rows past the end so that P = 0 there; delta 0
-            float v = (threadIdx.x < 32) ? (ok ? stat_reg * kLog2e : INFINITY) : (ok ? stat_reg : 0.f);
-            stat_lds[buf * 64 + threadIdx.x] = v;
+            float v = (threadIdx.x < kBwdBM) ? (ok ? stat_reg * kLog2e : INFINITY)
+                                             : (ok ? stat_reg : 0.f);
+            stat_lds[buf * 2 * kBwdBM + threadIdx.x] = v;
         }
     };
 
@@ -155,25 +159,140 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
     }
     __syncthreads();
 
-    // wavefront-uniform activity of 32-key slab w of this workgroup for the query tile at i0
-    auto slab_active = [&](int w, int i0) __attribute__((always_inline)) {
-        const int ks0 = k0 + 32 * w;
-        const int i_last = min(i0 + kBwdBM, a.sq) - 1;
-        if (ks0 >= a.sk) return false;
-        if (a.causal && ks0 > i_last) return false;
-        if (a.window > 0 && i0 - (ks0 + 31) >= a.window) return false;
+    // wavefront-uniform: does the 32-query half tile at ih0 see any key of this wavefront?
+    auto half_active = [&](int ih0) __attribute__((always_inline)) {
+        const int i_last = min(ih0 + 32, a.sq) - 1;
+        if (kw0 >= a.sk || ih0 >= a.sq) return false;
+        if (a.causal && kw0 > i_last) return false;
+        if (a.window > 0 && ih0 - (kw0 + 31) >= a.window) return false;
         return true;
     };
+    auto half_needs_mask = [&](int ih0) __attribute__((always_inline)) {
+        const int i_last = min(ih0 + 32, a.sq) - 1;
+        return (kw0 + 32 > a.sk) || (a.causal && kw0 + 31 > ih0) ||
+               (a.window > 0 && i_last - kw0 >= a.window);
+    };
 
-    TSTAMP();
-    // Iteration t: request tile t+1, do the S / dP / dV / dK work of tile t, write tile t+1 to LDS.
-    for (int t = t_lo; t < t_hi; ++t) {
+    // ---- stages of one half tile (32 queries at ih0 = i0 + 32 hf) ----
+    // S = Q_h K_w^T, dP = dO_h V_w^T
+    auto half_sp = [&](const T* qt, const T* gt, int hf, f32x16_t& s, f32x16_t& dp)
+                       __attribute__((always_inline)) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[r] = 0.f, dp[r] = 0.f;
+        const T* qrow = qt + 32 * hf * kPitch + a_off;
+        const T* grow = gt + 32 * hf * kPitch + a_off;
+#pragma unroll
+        for (int x = 0; x < DK; ++x) {
+            s = Mma<T>::mma32(lds_frag<T>(qrow + 16 * x), kf[x], s);
+            dp = Mma<T>::mma32(lds_frag<T>(grow + 16 * x), vf[x], dp);
+        }
+    };
+    // scores -> probabilities in place.  mask_tag: 0 = all visible, 1 = lower bound on the query
+    // only (causal / key tail), 2 = both bounds (local window)
+    auto half_exp = [&](f32x16_t& s, const float* lse_h, int ih0, auto mask_tag)
+                        __attribute__((always_inline)) {
+        constexpr int kMask = decltype(mask_tag)::value;
+        // register r is query ih0 + 8 g + c with c = acc_row(r, 0); visible iff c_lo <= c <= c_hi
+        int c_lo = 0, c_hi = 0;
+        if constexpr (kMask != 0) {
+            c_lo = (key < a.sk) ? (a.causal ? key - ih0 - 8 * g : -1) : 64;
+            if constexpr (kMask == 2) c_hi = key + a.window - 1 - ih0 - 8 * g;
+        }
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) {
+            const int qoff = acc_row(4 * r4, g);
+            const f32x4_t lse4 = *reinterpret_cast<const f32x4_t*>(lse_h + qoff);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                float x = __builtin_fmaf(s[4 * r4 + e], c_log2, -lse4[e]);
+                if constexpr (kBias) {
+                    const int i = ih0 + qoff + e;
+                    if (bias_per_key)
+                        x += bias_k;
+                    else if (i < a.sq && key < a.sk)
+                        x += a.bias[b * a.bs[0] + h * a.bs[1] + (int64_t)i * a.bs[2] +
+                                    (int64_t)key * a.bs[3]] * kLog2e;
+                }
+                float p = fast_exp2(x);
+                if constexpr (kMask != 0) {
+                    const int c = acc_row(4 * r4, 0) + e;
+                    if constexpr (kMask == 2) {
+                        if (c < c_lo || c > c_hi) p = 0.f;
+                    } else {
+                        if (c < c_lo) p = 0.f;
+                    }
+                }
+                s[4 * r4 + e] = p;
+            }
+        }
+    };
+    // P (after dropout) and dS = P (dP - delta), packed to T
+    auto half_ds = [&](const f32x16_t& p, const f32x16_t& dp, const float* delta_h, int ih0,
+                       uint32_t (&pw)[8], uint32_t (&dw)[8]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) {
+            const int qoff = acc_row(4 * r4, g);
+            const f32x4_t del4 = *reinterpret_cast<const f32x4_t*>(delta_h + qoff);
+            float pv[4], dv[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                float pe = p[4 * r4 + e];
+                float d = dp[4 * r4 + e];
+                float pd = pe;
+                if constexpr (kDropout) {
+                    const int i = ih0 + qoff + e;
+                    float keep = 0.f;
+                    if (i < a.sq && key < a.sk) {
+                        const uint64_t el =
+                            ((uint64_t)bh * a.sq + (uint64_t)i) * (uint64_t)a.sk + (uint64_t)key;
+                        bool kb;
+                        if (a.dropout_fast)
+                            kb = (dropout_keep4(a.rng, el >> 2) >> (el & 3)) & 1u;
+                        else
+                            kb = dropout_keep1(a.rng, el);
+                        keep = kb ? a.rng.inv_keep : 0.f;
+                    }
+                    pd = pe * keep;
+                    d = d * keep;
+                }
+                pv[e] = pd;
+                dv[e] = pe * (d - del4[e]);
+            }
+            pw[2 * r4] = pack2<T>(pv[0], pv[1]);
+            pw[2 * r4 + 1] = pack2<T>(pv[2], pv[3]);
+            dw[2 * r4] = pack2<T>(dv[0], dv[1]);
+            dw[2 * r4 + 1] = pack2<T>(dv[2], dv[3]);
+        }
+    };
+    // dV^T += dO_h^T P, dK^T += Q_h^T dS
+    auto half_out = [&](const T* qt, const T* gt, int hf, const uint32_t (&pw)[8],
+                        const uint32_t (&dw)[8]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh) {
+            u32x4_t pq = {pw[4 * hh], pw[4 * hh + 1], pw[4 * hh + 2], pw[4 * hh + 3]};
+            u32x4_t dq4 = {dw[4 * hh], dw[4 * hh + 1], dw[4 * hh + 2], dw[4 * hh + 3]};
+            const frag_t pf = __builtin_bit_cast(frag_t, pq);
+            const frag_t df = __builtin_bit_cast(frag_t, dq4);
+            const int off = (32 * hf + 16 * hh) * kPitch + t_off;
+#pragma unroll
+            for (int x = 0; x < DV; ++x) {
+                dv_acc[x] = Mma<T>::mma32(lds_frag_tr<T>(gt + off + 32 * x, kPitch), pf, dv_acc[x]);
+                dk_acc[x] = Mma<T>::mma32(lds_frag_tr<T>(qt + off + 32 * x, kPitch), df, dk_acc[x]);
+            }
+        }
+    };
+
+    // Iteration t: request tile t+1, process tile t, write tile t+1 into the other buffer.
+    // kFast iterations hold tiles in which every key of the workgroup sees every query, so their
+    // body is one straight block; the others test activity and masks per wavefront and half.
+    auto iteration = [&](int t, auto fast_tag) __attribute__((always_inline)) {
+        constexpr bool kFast = decltype(fast_tag)::value;
         TSTAMP();
         const int buf = (t - t_lo) & 1;
         const T* qt = q_lds + buf * SM::kQTile;
         const T* gt = g_lds + buf * SM::kQTile;
-        const float* lse_t = stat_lds + buf * 64;
-        const float* delta_t = lse_t + 32;
+        const float* lse_t = stat_lds + buf * 2 * kBwdBM;
+        const float* delta_t = lse_t + kBwdBM;
         const int i0 = t * kBwdBM;
         const bool have_next = t + 1 < t_hi;
         if (have_next) {
@@ -181,98 +300,36 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
             gst.load(g_base, a.os[1], i0 + kBwdBM, a.sq, a.d);
             load_stats(i0 + kBwdBM);
         }
-        const int i_last = min(i0 + kBwdBM, a.sq) - 1;
-        const bool active = slab_active(wave, i0);
-
-        auto tile_body = [&](auto mask_tag) __attribute__((always_inline)) {
-            constexpr bool kMask = decltype(mask_tag)::value;
-            // ---- S = Q K^T, dP = dO V^T ----
-            f32x16_t s_acc, p_acc;
+        if constexpr (kFast) {
+            std::integral_constant<int, 0> none;
+            f32x16_t s0, s1, p0, p1;
+            uint32_t pw0[8], dw0[8], pw1[8], dw1[8];
+            half_sp(qt, gt, 0, s0, p0);
+            half_exp(s0, lse_t, i0, none);
+            half_sp(qt, gt, 1, s1, p1);
+            half_ds(s0, p0, delta_t, i0, pw0, dw0);
+            half_exp(s1, lse_t + 32, i0 + 32, none);
+            half_out(qt, gt, 0, pw0, dw0);
+            half_ds(s1, p1, delta_t + 32, i0 + 32, pw1, dw1);
+            half_out(qt, gt, 1, pw1, dw1);
+        } else {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) s_acc[r] = 0.f, p_acc[r] = 0.f;
-            {
-                const T* qrow = qt + a_off;
-                const T* grow = gt + a_off;
-#pragma unroll
-                for (int x = 0; x < DK; ++x) {
-                    s_acc = Mma<T>::mma32(lds_frag<T>(qrow + 16 * x), kf[x], s_acc);
-                    p_acc = Mma<T>::mma32(lds_frag<T>(grow + 16 * x), vf[x], p_acc);
-                }
+            for (int hf = 0; hf < 2; ++hf) {
+                const int ih0 = i0 + 32 * hf;
+                if (!half_active(ih0)) continue;
+                f32x16_t s, dp;
+                uint32_t pw[8], dw[8];
+                half_sp(qt, gt, hf, s, dp);
+                if (!half_needs_mask(ih0))
+                    half_exp(s, lse_t + 32 * hf, ih0, std::integral_constant<int, 0>{});
+                else if (a.window > 0)
+                    half_exp(s, lse_t + 32 * hf, ih0, std::integral_constant<int, 2>{});
+                else
+                    half_exp(s, lse_t + 32 * hf, ih0, std::integral_constant<int, 1>{});
+                half_ds(s, dp, delta_t + 32 * hf, ih0, pw, dw);
+                half_out(qt, gt, hf, pw, dw);
             }
-            // ---- P and dS ----
-            uint32_t pw[8], dw[8];
-#pragma unroll
-            for (int r4 = 0; r4 < 4; ++r4) {
-                const int qoff = acc_row(4 * r4, g);
-                const f32x4_t lse4 = *reinterpret_cast<const f32x4_t*>(lse_t + qoff);
-                const f32x4_t del4 = *reinterpret_cast<const f32x4_t*>(delta_t + qoff);
-                float pv[4], dv[4];
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int i = i0 + qoff + e;
-                    float s = __builtin_fmaf(s_acc[4 * r4 + e], c_log2, -lse4[e]);
-                    if constexpr (kBias) {
-                        if (bias_per_key)
-                            s += bias_k;
-                        else if (i < a.sq && key < a.sk)
-                            s += a.bias[b * a.bs[0] + h * a.bs[1] + (int64_t)i * a.bs[2] +
-                                        (int64_t)key * a.bs[3]] * kLog2e;
-                    }
-                    float p = fast_exp2(s);
-                    if constexpr (kMask) {
-                        if (!key_visible(a, i, key)) p = 0.f;
-                    }
-                    float dp = p_acc[4 * r4 + e];
-                    float pd = p;
-                    if constexpr (kDropout) {
-                        float keep = 0.f;
-                        if (i < a.sq && key < a.sk) {
-                            const uint64_t el =
-                                ((uint64_t)bh * a.sq + (uint64_t)i) * (uint64_t)a.sk + (uint64_t)key;
-                            bool kb;
-                            if (a.dropout_fast)
-                                kb = (dropout_keep4(a.rng, el >> 2) >> (el & 3)) & 1u;
-                            else
-                                kb = dropout_keep1(a.rng, el);
-                            keep = kb ? a.rng.inv_keep : 0.f;
-                        }
-                        pd = p * keep;
-                        dp = dp * keep;
-                    }
-                    pv[e] = pd;
-                    dv[e] = p * (dp - del4[e]);
-                }
-                pw[2 * r4] = pack2<T>(pv[0], pv[1]);
-                pw[2 * r4 + 1] = pack2<T>(pv[2], pv[3]);
-                dw[2 * r4] = pack2<T>(dv[0], dv[1]);
-                dw[2 * r4 + 1] = pack2<T>(dv[2], dv[3]);
-            }
-            // ---- dV^T += dO^T P,  dK^T += Q^T dS ----
-#pragma unroll
-            for (int hh = 0; hh < 2; ++hh) {
-                u32x4_t pq = {pw[4 * hh], pw[4 * hh + 1], pw[4 * hh + 2], pw[4 * hh + 3]};
-                u32x4_t dq4 = {dw[4 * hh], dw[4 * hh + 1], dw[4 * hh + 2], dw[4 * hh + 3]};
-                const frag_t pf = __builtin_bit_cast(frag_t, pq);
-                const frag_t df = __builtin_bit_cast(frag_t, dq4);
-                const int off = 16 * hh * kPitch + t_off;
-#pragma unroll
-                for (int x = 0; x < DV; ++x) {
-                    dv_acc[x] =
-                        Mma<T>::mma32(lds_frag_tr<T>(gt + off + 32 * x, kPitch), pf, dv_acc[x]);
-                    dk_acc[x] =
-                        Mma<T>::mma32(lds_frag_tr<T>(qt + off + 32 * x, kPitch), df, dk_acc[x]);
-                }
-            }
-        };
-        if (active) {
-            const bool need_mask = (kw0 + 32 > a.sk) || (a.causal && kw0 + 31 > i0) ||
-                                   (a.window > 0 && i_last - kw0 >= a.window);
-            if (need_mask)
-                tile_body(std::true_type{});
-            else
-                tile_body(std::false_type{});
         }
-
         TSTAMP();
         // stage the next query tile (its buffer was last read before the previous barrier)
         if (have_next) {
@@ -285,6 +342,18 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
         TSTAMP();
         __syncthreads();
         TSTAMP();
+    };
+    auto tile_fast = [&](int t) __attribute__((always_inline)) {
+        const int i0 = t * kBwdBM;
+        return a.window <= 0 && k0 + kBwdBN <= a.sk && i0 + kBwdBM <= a.sq &&
+               (!a.causal || i0 >= k0 + kBwdBN - 1);
+    };
+    TSTAMP();
+    {
+        int t = t_lo;
+        for (; t < t_hi && !tile_fast(t); ++t) iteration(t, std::false_type{});
+        for (; t < t_hi && tile_fast(t); ++t) iteration(t, std::true_type{});
+        for (; t < t_hi; ++t) iteration(t, std::false_type{});
     }
 
     TSTAMP();
