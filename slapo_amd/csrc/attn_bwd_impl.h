@@ -313,10 +313,9 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
             half_ds(s1, p1, delta_t + 32, i0 + 32, pw1, dw1);
             half_out(qt, gt, 1, pw1, dw1);
         } else {
-#pragma unroll
-            for (int hf = 0; hf < 2; ++hf) {
+            auto generic_half = [&](int hf) __attribute__((always_inline)) {
                 const int ih0 = i0 + 32 * hf;
-                if (!half_active(ih0)) continue;
+                if (!half_active(ih0)) return;
                 f32x16_t s, dp;
                 uint32_t pw[8], dw[8];
                 half_sp(qt, gt, hf, s, dp);
@@ -328,7 +327,9 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
                     half_exp(s, lse_t + 32 * hf, ih0, std::integral_constant<int, 1>{});
                 half_ds(s, dp, delta_t + 32 * hf, ih0, pw, dw);
                 half_out(qt, gt, hf, pw, dw);
-            }
+            };
+            generic_half(0);
+            generic_half(1);
         }
         TSTAMP();
         // stage the next query tile (its buffer was last read before the previous barrier)

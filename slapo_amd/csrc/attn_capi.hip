@@ -132,7 +132,7 @@ bool half_ptrs_ok(std::initializer_list<const void*> ptrs) {
 
 }  // namespace
 
-#ifdef EXP_TIMING
+#if defined(EXP_TIMING) || defined(EXP_TIMING_DQ)
 void* g_timing_buf = nullptr;
 extern "C" int slapo_dbg_timing(unsigned long long* out, int n) {
     hipDeviceSynchronize();
@@ -234,7 +234,7 @@ extern "C" int slapo_amd_attn_bwd_stages(const slapo_attn_params* prm, const voi
     }
     // dK / dV (workgroups own keys), then dQ (workgroups own queries); both read delta.
     if (stages & SLAPO_BWD_DKDV) {
-#ifdef EXP_TIMING
+#if defined(EXP_TIMING) || defined(EXP_TIMING_DQ)
         if (!g_timing_buf) { hipMalloc(&g_timing_buf, 1 << 16); hipMemset(g_timing_buf, 0, 1 << 16); }
         a.o = g_timing_buf;
 #endif

@@ -173,16 +173,25 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_fwd_kerne
     };
 
     // bias, masks and tile maximum of freshly computed scores; returns the row maximum
+    // mask_tag: 0 = every key visible, 1 = upper bound only (causal / key tail), 2 = both bounds
     auto finish_scores = [&](f32x16_t (&s)[2], int t, auto mask_tag) __attribute__((always_inline)) -> float {
-        constexpr bool kMask = decltype(mask_tag)::value;
+        constexpr int kMask = decltype(mask_tag)::value;
         const int j0 = t * kBN;
+        // register (kb, r) is key j0 + 8 g + c with c = 32 kb + acc_row(r, 0); visible iff
+        // c_lo <= c <= c_hi
+        int c_lo = 0, c_hi = 0;
+        if constexpr (kMask != 0) {
+            const int k_max = a.causal ? min(a.sk - 1, q_row) : a.sk - 1;
+            c_hi = k_max - j0 - 8 * g;
+            if constexpr (kMask == 2) c_lo = q_row - a.window + 1 - j0 - 8 * g;
+        }
         float mx = -INFINITY;
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb) {
 #pragma unroll
             for (int r4 = 0; r4 < 4; ++r4) {
-                const int key0 = j0 + kb * 32 + acc_row(4 * r4, g);
                 if constexpr (kBias) {
+                    const int key0 = j0 + kb * 32 + acc_row(4 * r4, g);
                     float bv[4] = {0.f, 0.f, 0.f, 0.f};
                     if (a.bias_vec4 && key0 + 3 < a.sk) {
                         const f32x4_t t4 = *reinterpret_cast<const f32x4_t*>(bias_row + key0);
@@ -197,16 +206,27 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_fwd_kerne
                         s[kb][4 * r4 + e] =
                             __builtin_fmaf(s[kb][4 * r4 + e], c_log2, bv[e] * kLog2e);
                 }
-                if constexpr (kMask) {
+                if constexpr (kMask != 0) {
 #pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        if (!key_visible(a, q_row, key0 + e)) s[kb][4 * r4 + e] = -INFINITY;
+                    for (int e = 0; e < 4; ++e) {
+                        const int c = kb * 32 + acc_row(4 * r4, 0) + e;
+                        if constexpr (kMask == 2) {
+                            if (c > c_hi || c < c_lo) s[kb][4 * r4 + e] = -INFINITY;
+                        } else {
+                            if (c > c_hi) s[kb][4 * r4 + e] = -INFINITY;
+                        }
+                    }
                 }
                 mx = fmaxf(mx, fmaxf(fmaxf(s[kb][4 * r4], s[kb][4 * r4 + 1]),
                                      fmaxf(s[kb][4 * r4 + 2], s[kb][4 * r4 + 3])));
             }
         }
         return max_xor32(mx);
+    };
+    auto finish_any = [&](f32x16_t (&s)[2], int t) __attribute__((always_inline)) -> float {
+        if (!tile_needs_mask(t)) return finish_scores(s, t, std::integral_constant<int, 0>{});
+        if (a.window > 0) return finish_scores(s, t, std::integral_constant<int, 2>{});
+        return finish_scores(s, t, std::integral_constant<int, 1>{});
     };
 
     // move the reference point if this tile's maximum calls for it (rare after the first tile)
@@ -319,8 +339,7 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_fwd_kerne
     bool cur_active = tile_active(t_lo);
     if (cur_active) {
         scores(k_lds, s_a);
-        const float mx = tile_needs_mask(t_lo) ? finish_scores(s_a, t_lo, std::true_type{})
-                                               : finish_scores(s_a, t_lo, std::false_type{});
+        const float mx = finish_any(s_a, t_lo);
         update_reference(mx);
     }
     // K slot 0 is overwritten (with tile 2) at the end of iteration 0: every wavefront must have
@@ -348,15 +367,13 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_fwd_kerne
             scores(k_next, s_next);
             probabilities(s_cur, t, pw);
             accumulate(v_cur, pw);
-            mx_next = tile_needs_mask(t + 1) ? finish_scores(s_next, t + 1, std::true_type{})
-                                             : finish_scores(s_next, t + 1, std::false_type{});
+            mx_next = finish_any(s_next, t + 1);
         } else if (cur_active) {
             probabilities(s_cur, t, pw);
             accumulate(v_cur, pw);
         } else if (next_active) {
             scores(k_next, s_next);
-            mx_next = tile_needs_mask(t + 1) ? finish_scores(s_next, t + 1, std::true_type{})
-                                             : finish_scores(s_next, t + 1, std::false_type{});
+            mx_next = finish_any(s_next, t + 1);
         }
         if (next_active) update_reference(mx_next);
         cur_active = next_active;
