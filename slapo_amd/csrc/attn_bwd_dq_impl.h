@@ -30,7 +30,7 @@ constexpr int kBN = 64;
 constexpr int kKRing = 2;
 constexpr int kVRing = 2;
 
-template <typename T, int DPAD, bool kBias, bool kDropout>
+template <typename T, int DPAD, bool kBias, int kDrop>
 __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_dq_kernel(
     const AttnArgs a) {
     typedef typename Mma<T>::frag frag_t;
@@ -114,7 +114,7 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_dq_ke
     const int wq_last = min(wq0 + 31, a.sq - 1);
     const float c_log2 = a.scale_log2;
     uint64_t drop_row_base = 0;
-    if constexpr (kDropout)
+    if constexpr (kDrop != 0)
         drop_row_base = ((uint64_t)bh * a.sq + (uint64_t)q_row) * (uint64_t)a.sk;
     const float* bias_row = nullptr;
     if constexpr (kBias)
@@ -220,26 +220,22 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_dq_ke
 #pragma unroll
         for (int r4 = 0; r4 < 4; ++r4) {
             uint32_t bits = 0xFu;
-            if constexpr (kDropout) {
+            if constexpr (kDrop != 0) {
                 const int key0 = j0 + acc_row(4 * r4, g);
                 bits = 0;
                 if (q_row < a.sq && key0 < a.sk) {
                     const uint64_t e0 = drop_row_base + (uint64_t)key0;
-                    if (a.dropout_fast) {
-                        bits = dropout_keep4(a.rng, e0 >> 2);
-                    } else {
-#pragma unroll
-                        for (int e = 0; e < 4; ++e)
-                            if (key0 + e < a.sk)
-                                bits |= (dropout_keep1(a.rng, e0 + e) ? 1u : 0u) << e;
-                    }
+                    if constexpr (kDrop == 1)
+                        bits = dropout_keep4_pow2(a.rng, e0 >> 2);
+                    else
+                        bits = dropout_keep_any(a.rng, e0, min(4, a.sk - key0));
                 }
             }
             float dv[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 float d = dp[4 * r4 + e];
-                if constexpr (kDropout) d = ((bits >> e) & 1u) ? d * a.rng.inv_keep : 0.f;
+                if constexpr (kDrop != 0) d = ((bits >> e) & 1u) ? d * a.rng.inv_keep : 0.f;
                 dv[e] = p[4 * r4 + e] * (d - delta);
             }
             dw[2 * r4] = pack2<T>(dv[0], dv[1]);
@@ -259,6 +255,69 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_dq_ke
         half_dq(kt, 0, dw0);
         half_ds(s1, p1, t, 1, dw1);
         half_dq(kt, 1, dw1);
+    };
+
+    // Hand-scheduled version of tile_body for tiles without masks: the LDS operands of each group
+    // of matrix instructions are requested one phase before the group runs, and scheduling fences
+    // keep the compiler from sinking the requests back down to their uses.
+    auto tile_body_fast = [&](const T* kt, const T* vt, int t) __attribute__((always_inline)) {
+        std::integral_constant<int, 0> none;
+        frag_t kr0[DK], vr0[DK], kr1[DK], vr1[DK], kq0[2 * DV], kq1[2 * DV];
+        f32x16_t s0, s1, p0, p1;
+        uint32_t dw0[8], dw1[8];
+        auto rows = [&](const T* tile, int kb, frag_t (&f)[DK]) __attribute__((always_inline)) {
+#pragma unroll
+            for (int x = 0; x < DK; ++x)
+                f[x] = lds_frag<T>(tile + kb * 32 * kPitch + row_off + 16 * x);
+        };
+        auto cols = [&](int kb, frag_t (&f)[2 * DV]) __attribute__((always_inline)) {
+#pragma unroll
+            for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+                for (int x = 0; x < DV; ++x)
+                    f[s2 * DV + x] =
+                        lds_frag_tr<T>(kt + (32 * kb + 16 * s2) * kPitch + tr_off + 32 * x, kPitch);
+        };
+        auto mma_rows = [&](const frag_t (&f)[DK], const frag_t (&bfr)[DK], f32x16_t& acc)
+                            __attribute__((always_inline)) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+#pragma unroll
+            for (int x = 0; x < DK; ++x) acc = Mma<T>::mma32(f[x], bfr[x], acc);
+        };
+        auto mma_cols = [&](const frag_t (&f)[2 * DV], const uint32_t (&dw)[8])
+                            __attribute__((always_inline)) {
+#pragma unroll
+            for (int s2 = 0; s2 < 2; ++s2) {
+                u32x4_t dq4 = {dw[4 * s2], dw[4 * s2 + 1], dw[4 * s2 + 2], dw[4 * s2 + 3]};
+                const frag_t df = __builtin_bit_cast(frag_t, dq4);
+#pragma unroll
+                for (int x = 0; x < DV; ++x)
+                    dq_acc[x] = Mma<T>::mma32(f[s2 * DV + x], df, dq_acc[x]);
+            }
+        };
+        rows(kt, 0, kr0);
+        rows(vt, 0, vr0);
+        __builtin_amdgcn_sched_barrier(0);
+        rows(kt, 1, kr1);
+        mma_rows(kr0, qf, s0);
+        __builtin_amdgcn_sched_barrier(0);
+        rows(vt, 1, vr1);
+        mma_rows(vr0, gf, p0);
+        __builtin_amdgcn_sched_barrier(0);
+        cols(0, kq0);
+        mma_rows(kr1, qf, s1);
+        half_exp(s0, t, 0, none);
+        __builtin_amdgcn_sched_barrier(0);
+        cols(1, kq1);
+        mma_rows(vr1, gf, p1);
+        half_ds(s0, p0, t, 0, dw0);
+        __builtin_amdgcn_sched_barrier(0);
+        mma_cols(kq0, dw0);
+        half_exp(s1, t, 1, none);
+        half_ds(s1, p1, t, 1, dw1);
+        __builtin_amdgcn_sched_barrier(0);
+        mma_cols(kq1, dw1);
     };
 
     // ---- prologue: tile 0 into LDS ----
@@ -288,7 +347,11 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_dq_ke
         const T* kt = k_lds + (r % kKRing) * kTileElems;
         const T* vt = v_lds + (r % kVRing) * kTileElems;
         if constexpr (kFast) {
+#ifdef EXP_NO_HANDSCHED
             tile_body(kt, vt, t, std::integral_constant<int, 0>{});
+#else
+            tile_body_fast(kt, vt, t);
+#endif
         } else if (tile_active(t)) {
             if (!tile_needs_mask(t))
                 tile_body(kt, vt, t, std::integral_constant<int, 0>{});
@@ -339,14 +402,14 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_dq_ke
     }
 }
 
-template <typename T, int DPAD, bool kBias, bool kDropout>
+template <typename T, int DPAD, bool kBias, int kDrop>
 int launch(const AttnArgs& a, hipStream_t st) {
     typedef TileStage<T, DPAD, kBN, kThreads> Stage;
     const size_t smem = (size_t)(kKRing + kVRing) * kBN * Stage::kPitch * sizeof(T);
     const int n_qt = (a.sq + kBM - 1) / kBM;
     const int64_t blocks = (int64_t)n_qt * a.batch * a.heads;
     if (blocks <= 0 || blocks > 0x7FFFFFFF) return SLAPO_ERR_SHAPE;
-    auto kern = attn_bwd_dq_kernel<T, DPAD, kBias, kDropout>;
+    auto kern = attn_bwd_dq_kernel<T, DPAD, kBias, kDrop>;
     if (smem > 48 * 1024) {
         static bool raised = false;  // per instantiation
         if (!raised) {
@@ -364,11 +427,13 @@ int launch(const AttnArgs& a, hipStream_t st) {
 template <typename T, int DPAD>
 int dispatch_flags(const AttnArgs& a, hipStream_t st) {
     if (a.has_bias) {
-        if (a.dropout) return launch<T, DPAD, true, true>(a, st);
-        return launch<T, DPAD, true, false>(a, st);
+        if (a.dropout == 1) return launch<T, DPAD, true, 1>(a, st);
+        if (a.dropout == 2) return launch<T, DPAD, true, 2>(a, st);
+        return launch<T, DPAD, true, 0>(a, st);
     }
-    if (a.dropout) return launch<T, DPAD, false, true>(a, st);
-    return launch<T, DPAD, false, false>(a, st);
+    if (a.dropout == 1) return launch<T, DPAD, false, 1>(a, st);
+    if (a.dropout == 2) return launch<T, DPAD, false, 2>(a, st);
+    return launch<T, DPAD, false, 0>(a, st);
 }
 
 template <typename T>

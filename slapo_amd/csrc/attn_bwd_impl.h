@@ -43,7 +43,7 @@ struct BwdSmem {
     static constexpr size_t kBytes = 2 * kQBytes + kStatBytes;
 };
 
-template <typename T, int DPAD, bool kBias, bool kDropout>
+template <typename T, int DPAD, bool kBias, int kDrop>
 __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_kernel(
     const AttnArgs a) {
     typedef typename Mma<T>::frag frag_t;
@@ -229,6 +229,41 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
     // P (after dropout) and dS = P (dP - delta), packed to T
     auto half_ds = [&](const f32x16_t& p, const f32x16_t& dp, const float* delta_h, int ih0,
                        uint32_t (&pw)[8], uint32_t (&dw)[8]) __attribute__((always_inline)) {
+        // Keep-bits of this half: wq[e] bit 4 * r4 belongs to register 4 * r4 + e.
+        uint32_t wq[4] = {0u, 0u, 0u, 0u};
+        if constexpr (kDrop == 1) {
+            // The four lanes of a quad hold four consecutive keys, i.e. one Philox block per query
+            // row.  Lane j of the quad draws the blocks of the rows held in registers j, j+4, j+8,
+            // j+12 and the quad exchanges them: 4 blocks per lane instead of 16.
+            const int qpos = lane & 3;
+            uint32_t mine = 0;
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                const int i = ih0 + acc_row(4 * r4, g) + qpos;
+                if (i < a.sq && key < a.sk) {
+                    const uint64_t el =
+                        ((uint64_t)bh * a.sq + (uint64_t)i) * (uint64_t)a.sk + (uint64_t)(key & ~3);
+                    mine |= dropout_keep4_pow2(a.rng, el >> 2) << (4 * r4);
+                }
+            }
+            wq[0] = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)mine, 0x00, 0xF, 0xF, false) >> qpos;
+            wq[1] = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)mine, 0x55, 0xF, 0xF, false) >> qpos;
+            wq[2] = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)mine, 0xAA, 0xF, 0xF, false) >> qpos;
+            wq[3] = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)mine, 0xFF, 0xF, 0xF, false) >> qpos;
+        } else if constexpr (kDrop == 2) {
+            uint32_t mask16 = 0;  // bit r <-> register r
+#pragma unroll 1
+            for (int r = 0; r < 16; ++r) {
+                const int i = ih0 + acc_row(r, g);
+                if (i < a.sq && key < a.sk) {
+                    const uint64_t el =
+                        ((uint64_t)bh * a.sq + (uint64_t)i) * (uint64_t)a.sk + (uint64_t)key;
+                    if (dropout_keep1(a.rng, el)) mask16 |= 1u << r;
+                }
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) wq[e] = mask16 >> e;
+        }
 #pragma unroll
         for (int r4 = 0; r4 < 4; ++r4) {
             const int qoff = acc_row(4 * r4, g);
@@ -239,19 +274,8 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
                 float pe = p[4 * r4 + e];
                 float d = dp[4 * r4 + e];
                 float pd = pe;
-                if constexpr (kDropout) {
-                    const int i = ih0 + qoff + e;
-                    float keep = 0.f;
-                    if (i < a.sq && key < a.sk) {
-                        const uint64_t el =
-                            ((uint64_t)bh * a.sq + (uint64_t)i) * (uint64_t)a.sk + (uint64_t)key;
-                        bool kb;
-                        if (a.dropout_fast)
-                            kb = (dropout_keep4(a.rng, el >> 2) >> (el & 3)) & 1u;
-                        else
-                            kb = dropout_keep1(a.rng, el);
-                        keep = kb ? a.rng.inv_keep : 0.f;
-                    }
+                if constexpr (kDrop != 0) {
+                    const float keep = ((wq[e] >> (4 * r4)) & 1u) ? a.rng.inv_keep : 0.f;
                     pd = pe * keep;
                     d = d * keep;
                 }
@@ -380,14 +404,14 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
     }
 }
 
-template <typename T, int DPAD, bool kBias, bool kDropout>
+template <typename T, int DPAD, bool kBias, int kDrop>
 int launch(const AttnArgs& a, hipStream_t st) {
     typedef BwdSmem<T, DPAD> SM;
     const size_t smem = SM::kBytes;
     const int n_kt = (a.sk + kBwdBN - 1) / kBwdBN;
     const int64_t blocks = (int64_t)n_kt * a.batch * a.heads;
     if (blocks <= 0 || blocks > 0x7FFFFFFF) return SLAPO_ERR_SHAPE;
-    auto kern = attn_bwd_kernel<T, DPAD, kBias, kDropout>;
+    auto kern = attn_bwd_kernel<T, DPAD, kBias, kDrop>;
     if (smem > 48 * 1024) {
         static bool raised = false;  // per instantiation
         if (!raised) {
@@ -418,11 +442,13 @@ int launch(const AttnArgs& a, hipStream_t st) {
 template <typename T, int DPAD>
 int dispatch_flags(const AttnArgs& a, hipStream_t st) {
     if (a.has_bias) {
-        if (a.dropout) return launch<T, DPAD, true, true>(a, st);
-        return launch<T, DPAD, true, false>(a, st);
+        if (a.dropout == 1) return launch<T, DPAD, true, 1>(a, st);
+        if (a.dropout == 2) return launch<T, DPAD, true, 2>(a, st);
+        return launch<T, DPAD, true, 0>(a, st);
     }
-    if (a.dropout) return launch<T, DPAD, false, true>(a, st);
-    return launch<T, DPAD, false, false>(a, st);
+    if (a.dropout == 1) return launch<T, DPAD, false, 1>(a, st);
+    if (a.dropout == 2) return launch<T, DPAD, false, 2>(a, st);
+    return launch<T, DPAD, false, 0>(a, st);
 }
 
 template <typename T>

@@ -102,12 +102,11 @@ int fill_args(const slapo_attn_params* p, AttnArgs* a, bool backward) {
     a->scale = p->scale;
     a->scale_log2 = p->scale * kLog2e;
     a->dropout = p->p_drop > 0.f ? 1 : 0;
-    a->dropout_fast = 0;
     if (a->dropout) {
         const int64_t numel = (int64_t)p->batch * p->heads * p->seqlen_q * p->seqlen_k;
         if (!plan_ok(&p->plan, numel)) return SLAPO_ERR_ARG;
         a->rng = make_dropout_state(p->plan, (double)p->p_drop, p->seed, p->offset);
-        a->dropout_fast = (p->plan.vec >= 4 && p->seqlen_k % 4 == 0) ? 1 : 0;
+        if (!(a->rng.g_shift >= 0 && a->rng.t_shift >= 0 && p->seqlen_k % 4 == 0)) a->dropout = 2;
     } else {
         a->rng = DropoutState{};
     }

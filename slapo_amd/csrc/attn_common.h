@@ -133,7 +133,9 @@ struct AttnArgs {
     int batch, heads, sq, sk, d;
     int causal, window;
     int has_bias, bias_vec4;  // bias_vec4: s3 == 1, s2 == 0 rows 16B-aligned
-    int dropout, dropout_fast;  // dropout_fast: plan.vec >= 4 and sk % 4 == 0
+    // dropout: 0 = off, 1 = fast mask geometry (plan.vec >= 4, power-of-two thread count and
+    // sk % 4 == 0: one Philox block per aligned group of four keys), 2 = any geometry
+    int dropout;
     float scale, scale_log2;
     DropoutState rng;
 };

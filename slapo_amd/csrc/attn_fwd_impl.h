@@ -49,7 +49,7 @@ constexpr int kVRing = 3;
 // normalisation, well inside fp16 / fp32 range.
 constexpr float kMaxSlack = 8.0f;
 
-template <typename T, int DPAD, bool kBias, bool kDropout>
+template <typename T, int DPAD, bool kBias, int kDrop>
 __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_fwd_kernel(
     const AttnArgs a) {
     typedef typename Mma<T>::frag frag_t;
@@ -128,7 +128,7 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_fwd_kerne
     const float c_log2 = a.scale_log2;
     const float slack = kBias ? kMaxSlack : kMaxSlack / c_log2;
     uint64_t drop_row_base = 0;
-    if constexpr (kDropout)
+    if constexpr (kDrop != 0)
         drop_row_base = ((uint64_t)bh * a.sq + (uint64_t)q_row) * (uint64_t)a.sk;
     const float* bias_row = nullptr;
     if constexpr (kBias)
@@ -265,7 +265,7 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_fwd_kerne
                 psum += p;
             }
         l_run += psum;
-        if constexpr (kDropout) {
+        if constexpr (kDrop != 0) {
             const int j0 = t * kBN;
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
@@ -275,14 +275,10 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_fwd_kerne
                     uint32_t bits = 0;
                     if (q_row < a.sq && key0 < a.sk) {
                         const uint64_t e0 = drop_row_base + (uint64_t)key0;
-                        if (a.dropout_fast) {
-                            bits = dropout_keep4(a.rng, e0 >> 2);
-                        } else {
-#pragma unroll
-                            for (int e = 0; e < 4; ++e)
-                                if (key0 + e < a.sk)
-                                    bits |= (dropout_keep1(a.rng, e0 + e) ? 1u : 0u) << e;
-                        }
+                        if constexpr (kDrop == 1)
+                            bits = dropout_keep4_pow2(a.rng, e0 >> 2);
+                        else
+                            bits = dropout_keep_any(a.rng, e0, min(4, a.sk - key0));
                     }
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
@@ -420,14 +416,14 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_fwd_kerne
     }
 }
 
-template <typename T, int DPAD, bool kBias, bool kDropout>
+template <typename T, int DPAD, bool kBias, int kDrop>
 int launch(const AttnArgs& a, hipStream_t st) {
     typedef TileStage<T, DPAD, kBN, kThreads> Stage;
     const size_t smem = (size_t)(kKRing + kVRing) * kBN * Stage::kPitch * sizeof(T);
     const int n_qt = (a.sq + kBM - 1) / kBM;
     const int64_t blocks = (int64_t)n_qt * a.batch * a.heads;
     if (blocks <= 0 || blocks > 0x7FFFFFFF) return SLAPO_ERR_SHAPE;
-    auto kern = attn_fwd_kernel<T, DPAD, kBias, kDropout>;
+    auto kern = attn_fwd_kernel<T, DPAD, kBias, kDrop>;
     if (smem > 48 * 1024) {
         static bool raised = false;  // per instantiation
         if (!raised) {
@@ -445,11 +441,13 @@ int launch(const AttnArgs& a, hipStream_t st) {
 template <typename T, int DPAD>
 int dispatch_flags(const AttnArgs& a, hipStream_t st) {
     if (a.has_bias) {
-        if (a.dropout) return launch<T, DPAD, true, true>(a, st);
-        return launch<T, DPAD, true, false>(a, st);
+        if (a.dropout == 1) return launch<T, DPAD, true, 1>(a, st);
+        if (a.dropout == 2) return launch<T, DPAD, true, 2>(a, st);
+        return launch<T, DPAD, true, 0>(a, st);
     }
-    if (a.dropout) return launch<T, DPAD, false, true>(a, st);
-    return launch<T, DPAD, false, false>(a, st);
+    if (a.dropout == 1) return launch<T, DPAD, false, 1>(a, st);
+    if (a.dropout == 2) return launch<T, DPAD, false, 2>(a, st);
+    return launch<T, DPAD, false, 0>(a, st);
 }
 
 template <typename T>

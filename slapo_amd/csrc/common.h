@@ -101,6 +101,7 @@ inline DropoutState make_dropout_state(const slapo_dropout_plan& plan, double p,
         while ((1ull << sh) != s.total_threads) ++sh;
         s.t_shift = sh;
     }
+    s.g_shift = s.vec >= 4 ? (s.vec == 4 ? 0 : s.vec == 8 ? 1 : 2) : -1;
     s.inv_keep = p < 1.0 ? (float)(1.0 / (double)(float)(1.0 - p)) : 0.f;
     return s;
 }

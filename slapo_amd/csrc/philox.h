@@ -59,6 +59,7 @@ struct DropoutState {
     uint32_t keep_max;        // keep iff word <= keep_max (unless keep_none)
     uint32_t keep_none;       // 1: nothing is kept (p == 1)
     int32_t t_shift;          // log2(T) when T is a power of two, else -1
+    int32_t g_shift;          // log2(vec / 4) when vec >= 4, else -1
     float inv_keep;           // 1 / (1 - p)
 };
 
@@ -124,6 +125,29 @@ SLAPO_HD uint32_t dropout_keep4(const DropoutState& s, uint64_t group) {
     const u32x4 r = philox_block(s, thread, trip * s.calls_per_iter + sub);
     return (keep_word(s, r.x) ? 1u : 0u) | (keep_word(s, r.y) ? 2u : 0u) |
            (keep_word(s, r.z) ? 4u : 0u) | (keep_word(s, r.w) ? 8u : 0u);
+}
+
+// dropout_keep4 for the common launch geometry: vec >= 4 and a power-of-two thread count, so the
+// element -> (subsequence, counter) split is shifts and masks only.
+SLAPO_HD uint32_t dropout_keep4_pow2(const DropoutState& s, uint64_t group) {
+    const uint64_t v = group >> s.g_shift;
+    const uint32_t sub = (uint32_t)group & ((1u << s.g_shift) - 1u);
+    const uint64_t thread = v & (s.total_threads - 1);
+    const uint64_t trip = v >> s.t_shift;
+    const u32x4 r = philox_block(s, thread, trip * s.calls_per_iter + sub);
+    return (keep_word(s, r.x) ? 1u : 0u) | (keep_word(s, r.y) ? 2u : 0u) |
+           (keep_word(s, r.z) ? 4u : 0u) | (keep_word(s, r.w) ? 8u : 0u);
+}
+
+// Keep-bits of the n (1..4) consecutive elements starting at elem, for any launch geometry and
+// alignment.  Deliberately a rolled loop: this path is rare and must stay small.
+SLAPO_HD uint32_t dropout_keep_any(const DropoutState& s, uint64_t elem, int n) {
+    uint32_t bits = 0;
+#if defined(__HIPCC__)
+#pragma unroll 1
+#endif
+    for (int e = 0; e < n; ++e) bits |= (dropout_keep1(s, elem + (uint64_t)e) ? 1u : 0u) << e;
+    return bits;
 }
 
 }  // namespace slapo
