@@ -7,9 +7,10 @@ Q/K/V/dO ~ N(0,1) from seed 2013 (synthetic).  All tensors are resident in HBM b
 region; the kernels are called through the C ABI (libslapo_amd.so) with preallocated outputs.
 
 value     attention fwd+bwd TFLOP/s = 14 * D * N / time per step, N = attended (query, key) pairs
-roofline  the backward MFMA kernel (the dominant kernel): its algorithmic FLOPs (10 * D * N) over
-          its own average launch duration, taken with HIP events placed around the MAIN stage of
-          the backward on the launching stream, against the dense fp16 MFMA peak
+roofline  the dK/dV backward kernel (the dominant kernel): its algorithmic FLOPs (8 * D * N: the
+          four matrix products S, dP, dV, dK) over its own average launch duration, taken with HIP
+          events placed around the DKDV stage of the backward on the launching stream, against the
+          dense fp16 MFMA peak; "kernels" lists the same figure for the forward and dQ kernels
 epilogue  GB/s of the two FusedMLP epilogues (bf16, tokens 8192, 1024 -> 4096 -> 1024) against the
           HBM peak, on a rotating working set larger than the caches
 cpu_baseline  the oracle's native-PyTorch restatement (fp32 CPU, autograd backward) timed on the
@@ -31,6 +32,11 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 / bf16
+# HBM bytes per launch of the dK/dV kernel on WORKLOAD, from rocprofv3 --pmc FETCH_SIZE and
+# WRITE_SIZE (KiB per dispatch), each scaled by the same counter's reading for a 256 MiB copy
+# (FETCH_SIZE reads half the copied bytes: factor 2.0; WRITE_SIZE factor 1.0):
+# (51.75e3 * 2.0 + 67.09e3) KiB.  Summary under profiles/.
+DKDV_TRAFFIC_BYTES = (51.75e3 * 2.0 + 67.09e3) * 1024
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 
 WORKLOAD = dict(name="gpt2-medium causal attention fwd+bwd", dtype="fp16", batch=8, seq=1024,
@@ -87,14 +93,21 @@ class AttentionStep:
             raise RuntimeError(f"slapo_amd_attn_bwd_stages failed with status {rc}")
 
     def step(self, ev=None):
-        self.forward()
-        self.backward(self._lib_mod.BWD_PREPARE)
+        """ev: five events recorded around forward | prepare | dK/dV | dQ."""
         if ev is not None:
             ev[0].record()
-        self.backward(self._lib_mod.BWD_DKDV)
+        self.forward()
         if ev is not None:
             ev[1].record()
+        self.backward(self._lib_mod.BWD_PREPARE)
+        if ev is not None:
+            ev[2].record()
+        self.backward(self._lib_mod.BWD_DKDV)
+        if ev is not None:
+            ev[3].record()
         self.backward(self._lib_mod.BWD_DQ)
+        if ev is not None:
+            ev[4].record()
 
 
 def bench_epilogues(device, iters=40):
@@ -203,6 +216,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-epilogues", action="store_true")
+    ap.add_argument("--traffic-reference", action="store_true",
+                    help="also run three 256 MiB device-to-device copies, the known-size kernel "
+                         "against which FETCH_SIZE / WRITE_SIZE counter readings are scaled")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU's throughput; --gpus above 1 is not supported "
@@ -213,12 +229,19 @@ def main():
     cfg = WORKLOAD
     device = torch.device("cuda", 0)
     torch.cuda.set_device(device)
+    if args.traffic_reference:
+        src = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device=device).normal_()
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     step = AttentionStep(cfg, device)
 
     for _ in range(args.warmup):
         step.step()
     torch.cuda.synchronize()
-    events = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True))
+    events = [[torch.cuda.Event(enable_timing=True) for _ in range(5)]
               for _ in range(args.steps)]
     t0 = time.perf_counter()
     for i in range(args.steps):
@@ -230,9 +253,15 @@ def main():
     d = cfg["head_dim"]
     ms_per_step = elapsed / args.steps * 1e3
     value = 14 * d * n_pairs / (elapsed / args.steps) / 1e12
-    kern_ms = sum(a.elapsed_time(b) for a, b in events) / args.steps
-    bwd_flops = 10 * d * n_pairs
+    seg_ms = [sum(ev[i].elapsed_time(ev[i + 1]) for ev in events) / args.steps for i in range(4)]
+    kern_ms = seg_ms[2]
+    bwd_flops = 8 * d * n_pairs
     achieved = bwd_flops / (kern_ms * 1e-3) / 1e12
+
+    def kern(name, flops, ms):
+        tf = flops / (ms * 1e-3) / 1e12
+        return {"kernel": name, "flops_per_launch": flops, "avg_launch_ms": ms, "TFLOPs": tf,
+                "frac_of_mfma_peak": tf / MFMA_PEAK_TFLOPS}
 
     result = {
         "metric": "attention fwd+bwd TFLOP/s + epilogue GB/s, % of MI355X roofline, 1 GPU",
@@ -251,11 +280,16 @@ def main():
                    "heads": cfg["heads"], "head_dim": cfg["head_dim"], "causal": cfg["causal"],
                    "dropout_p": cfg["p"], "flops_per_step": 14 * d * n_pairs},
         "frac_of_mfma_peak": value / MFMA_PEAK_TFLOPS,
-        "roofline": {"bound": "mfma", "kernel": "attn_bwd_kernel<f16, 64>", "achieved": achieved,
+        "roofline": {"bound": "mfma", "kernel": "attn_bwd_kernel<f16, 64, false, 0> (dK/dV)",
+                     "achieved": achieved,
                      "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / MFMA_PEAK_TFLOPS, "traffic": None,
+                     "frac": achieved / MFMA_PEAK_TFLOPS, "traffic": DKDV_TRAFFIC_BYTES,
                      "flops_per_launch": bwd_flops, "avg_launch_ms": kern_ms},
     }
+    result["kernels"] = [kern("attn_fwd_kernel<f16, 64, false, 0>", 4 * d * n_pairs, seg_ms[0]),
+                         kern("attn_bwd_kernel<f16, 64, false, 0> (dK/dV)", bwd_flops, seg_ms[2]),
+                         kern("attn_bwd_dq_kernel<f16, 64, false, 0>", 6 * d * n_pairs, seg_ms[3])]
+    result["delta_kernel_ms"] = seg_ms[1]
     if not args.no_epilogues:
         result["epilogue"] = bench_epilogues(device)
     if not args.no_cpu_baseline:

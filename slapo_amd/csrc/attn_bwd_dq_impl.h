@@ -74,29 +74,41 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_dq_ke
     const T* v_base = reinterpret_cast<const T*>(a.v) + b * a.vs[0] + h * a.vs[2];
     const T* g_base = reinterpret_cast<const T*>(a.dout) + b * a.os[0] + h * a.os[2];
 
-    // Q^T and dO^T fragments: column i = this lane's query, k-slots = 8 head-dim elements.
+    // Start-up loads, all issued before any of them is used: the Q^T and dO^T fragments (column
+    // i = this lane's query, k-slots = 8 head-dim elements), lse, delta and the first K / V tile.
+    // Addresses are clamped into the tensor; what was clamped is zeroed afterwards.
+    Stage ks, vs;
+    int j_lo, j_hi;
+    key_range(a, q0, min(q0 + kBM, a.sq), j_lo, j_hi);
+    const int t_lo = j_lo / kBN;
+    const int t_hi = (j_hi + kBN - 1) / kBN;
+    const int n_tiles = t_hi - t_lo;
+
     frag_t qf[DK], gf[DK];
-    float lse2 = INFINITY;  // log2 units; +inf for rows past the end so that P = 0 there
-    float delta = 0.f;
+    float lse2, delta;
     {
         const int qr = min(q_row, a.sq - 1);
+        u32x4_t qv[DK], gv[DK];
 #pragma unroll
         for (int t = 0; t < DK; ++t) {
-            const int d0 = 16 * t + 8 * g;
-            const int dc = min(d0, a.d - 8);
-            u32x4_t qv = *reinterpret_cast<const u32x4_t*>(q_base + (int64_t)qr * a.qs[1] + dc);
-            u32x4_t gv = *reinterpret_cast<const u32x4_t*>(g_base + (int64_t)qr * a.os[1] + dc);
-            if (q_row >= a.sq || d0 >= a.d) {
-                qv = u32x4_t{0u, 0u, 0u, 0u};
-                gv = u32x4_t{0u, 0u, 0u, 0u};
-            }
-            qf[t] = __builtin_bit_cast(frag_t, qv);
-            gf[t] = __builtin_bit_cast(frag_t, gv);
+            const int dc = min(16 * t + 8 * g, a.d - 8);
+            qv[t] = *reinterpret_cast<const u32x4_t*>(q_base + (int64_t)qr * a.qs[1] + dc);
+            gv[t] = *reinterpret_cast<const u32x4_t*>(g_base + (int64_t)qr * a.os[1] + dc);
         }
-        if (q_row < a.sq) {
-            lse2 = a.lse[(int64_t)bh * a.sq + q_row] * kLog2e;
-            delta = a.delta[(int64_t)bh * a.sq + q_row];
+        const float lse_raw = a.lse[(int64_t)bh * a.sq + qr];
+        const float delta_raw = a.delta[(int64_t)bh * a.sq + qr];
+        ks.load(k_base, a.ks[1], t_lo * kBN, a.sk, a.d);
+        vs.load(v_base, a.vs[1], t_lo * kBN, a.sk, a.d);
+        const bool row_ok = q_row < a.sq;
+#pragma unroll
+        for (int t = 0; t < DK; ++t) {
+            const bool keep = row_ok && (16 * t + 8 * g < a.d);
+            qf[t] = __builtin_bit_cast(frag_t, keep_or_zero(qv[t], keep));
+            gf[t] = __builtin_bit_cast(frag_t, keep_or_zero(gv[t], keep));
         }
+        // log2 units; +inf for rows past the end so that P = 0 there
+        lse2 = row_ok ? lse_raw * kLog2e : INFINITY;
+        delta = row_ok ? delta_raw : 0.f;
     }
 
     f32x16_t dq_acc[DV];
@@ -104,12 +116,6 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_dq_ke
     for (int x = 0; x < DV; ++x)
 #pragma unroll
         for (int r = 0; r < 16; ++r) dq_acc[x][r] = 0.f;
-
-    int j_lo, j_hi;
-    key_range(a, q0, min(q0 + kBM, a.sq), j_lo, j_hi);
-    const int t_lo = j_lo / kBN;
-    const int t_hi = (j_hi + kBN - 1) / kBN;
-    const int n_tiles = t_hi - t_lo;
 
     const int wq_last = min(wq0 + 31, a.sq - 1);
     const float c_log2 = a.scale_log2;
@@ -321,10 +327,7 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_dq_ke
     };
 
     // ---- prologue: tile 0 into LDS ----
-    Stage ks, vs;
     if (n_tiles > 0) {
-        ks.load(k_base, a.ks[1], t_lo * kBN, a.sk, a.d);
-        vs.load(v_base, a.vs[1], t_lo * kBN, a.sk, a.d);
         ks.fix(t_lo * kBN, a.sk, a.d);
         vs.fix(t_lo * kBN, a.sk, a.d);
         ks.store(k_lds);

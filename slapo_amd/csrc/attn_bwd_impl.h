@@ -92,18 +92,20 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
     const float* delta_base = a.delta + (int64_t)bh * a.sq;
 
     // ---- resident fragments ----
+    // Loaded with clamped addresses and masked once the first query tile has been requested too,
+    // so that all start-up loads of the workgroup are in flight together.
     frag_t kf[DK], vf[DK];
+    u32x4_t k_raw[DK], v_raw[DK];
+    {
+        const int kr = min(key, a.sk - 1);
 #pragma unroll
-    for (int t = 0; t < DK; ++t) {
-        u32x4_t kv = {0u, 0u, 0u, 0u}, vv = {0u, 0u, 0u, 0u};
-        const int d0 = 16 * t + 8 * g;
-        if (key < a.sk && d0 < a.d) {
-            kv = *reinterpret_cast<const u32x4_t*>(k_base + (int64_t)key * a.ks[1] + d0);
-            vv = *reinterpret_cast<const u32x4_t*>(v_base + (int64_t)key * a.vs[1] + d0);
+        for (int t = 0; t < DK; ++t) {
+            const int dc = min(16 * t + 8 * g, a.d - 8);
+            k_raw[t] = *reinterpret_cast<const u32x4_t*>(k_base + (int64_t)kr * a.ks[1] + dc);
+            v_raw[t] = *reinterpret_cast<const u32x4_t*>(v_base + (int64_t)kr * a.vs[1] + dc);
         }
-        kf[t] = __builtin_bit_cast(frag_t, kv);
-        vf[t] = __builtin_bit_cast(frag_t, vv);
     }
+
     f32x16_t dk_acc[DV], dv_acc[DV];
 #pragma unroll
     for (int x = 0; x < DV; ++x)
@@ -147,10 +149,17 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
         }
     };
 
+    // rows are clamped into the tensor, so the request is safe even without any query tile
+    qst.load(q_base, a.qs[1], t_lo * kBwdBM, a.sq, a.d);
+    gst.load(g_base, a.os[1], t_lo * kBwdBM, a.sq, a.d);
+    load_stats(t_lo * kBwdBM);
+#pragma unroll
+    for (int t = 0; t < DK; ++t) {
+        const bool keep = key < a.sk && 16 * t + 8 * g < a.d;
+        kf[t] = __builtin_bit_cast(frag_t, keep_or_zero(k_raw[t], keep));
+        vf[t] = __builtin_bit_cast(frag_t, keep_or_zero(v_raw[t], keep));
+    }
     if (t_lo < t_hi) {
-        qst.load(q_base, a.qs[1], t_lo * kBwdBM, a.sq, a.d);
-        gst.load(g_base, a.os[1], t_lo * kBwdBM, a.sq, a.d);
-        load_stats(t_lo * kBwdBM);
         qst.fix(t_lo * kBwdBM, a.sq, a.d);
         gst.fix(t_lo * kBwdBM, a.sq, a.d);
         qst.store(q_lds);

@@ -115,6 +115,14 @@ __device__ __forceinline__ float sum_xor32(float v) {
     return a + b;
 }
 
+// 16 bytes of a row fragment, or zeros when `keep` is false.  Written as a mask so that it stays
+// straight-line code: a branch here would make the compiler wait for the load on the spot, and
+// the start-up loads of a workgroup must all be in flight together.
+__device__ __forceinline__ u32x4_t keep_or_zero(u32x4_t v, bool keep) {
+    const uint32_t m = keep ? 0xFFFFFFFFu : 0u;
+    return u32x4_t{v.x & m, v.y & m, v.z & m, v.w & m};
+}
+
 // Kernel argument block (filled by the host dispatcher from slapo_attn_params).
 struct AttnArgs {
     const void* q;

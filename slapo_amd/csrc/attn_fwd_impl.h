@@ -93,17 +93,16 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_fwd_kerne
     const T* v_base = reinterpret_cast<const T*>(a.v) + b * a.vs[0] + h * a.vs[2];
 
     // Q^T fragments: column i = this lane's query, k-slots = 8 consecutive head-dim elements.
+    // The loads are issued here and masked after the first K / V tile loads have been issued too,
+    // so that all start-up loads of the workgroup are in flight together.
     frag_t qf[DK];
+    u32x4_t q_raw[DK];
     {
         const int qr = min(q_row, a.sq - 1);
 #pragma unroll
-        for (int t = 0; t < DK; ++t) {
-            const int d0 = 16 * t + 8 * g;
-            u32x4_t v = *reinterpret_cast<const u32x4_t*>(q_base + (int64_t)qr * a.qs[1] +
-                                                          min(d0, a.d - 8));
-            if (q_row >= a.sq || d0 >= a.d) v = u32x4_t{0u, 0u, 0u, 0u};
-            qf[t] = __builtin_bit_cast(frag_t, v);
-        }
+        for (int t = 0; t < DK; ++t)
+            q_raw[t] = *reinterpret_cast<const u32x4_t*>(q_base + (int64_t)qr * a.qs[1] +
+                                                         min(16 * t + 8 * g, a.d - 8));
     }
 
     f32x16_t o_acc[DV];
@@ -311,18 +310,25 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_fwd_kerne
     // Two register stages alternate: a tile is requested two iterations before it is written to
     // LDS, so a full iteration of math sits between the request and the wait.
     Stage ks_a, vs_a, ks_b, vs_b;
-#pragma unroll
-    for (int r = 0; r < 2; ++r) {
-        if (r < n_tiles) {
-            const int j0 = (t_lo + r) * kBN;
-            ks_a.load(k_base, a.ks[1], j0, a.sk, a.d);
-            vs_a.load(v_base, a.vs[1], j0, a.sk, a.d);
-            ks_a.fix(j0, a.sk, a.d);
-            vs_a.fix(j0, a.sk, a.d);
-            ks_a.store(k_lds + r * kTileElems);
-            vs_a.store(v_lds + r * kTileElems);
-        }
+    // rows are clamped into the tensor, so the requests are safe whatever n_tiles is
+    ks_a.load(k_base, a.ks[1], t_lo * kBN, a.sk, a.d);
+    vs_a.load(v_base, a.vs[1], t_lo * kBN, a.sk, a.d);
+    ks_b.load(k_base, a.ks[1], (t_lo + 1) * kBN, a.sk, a.d);
+    vs_b.load(v_base, a.vs[1], (t_lo + 1) * kBN, a.sk, a.d);
+    ks_a.fix(t_lo * kBN, a.sk, a.d);
+    vs_a.fix(t_lo * kBN, a.sk, a.d);
+    ks_a.store(k_lds);
+    vs_a.store(v_lds);
+    if (1 < n_tiles) {
+        ks_b.fix((t_lo + 1) * kBN, a.sk, a.d);
+        vs_b.fix((t_lo + 1) * kBN, a.sk, a.d);
+        ks_b.store(k_lds + kTileElems);
+        vs_b.store(v_lds + kTileElems);
     }
+#pragma unroll
+    for (int t = 0; t < DK; ++t)
+        qf[t] = __builtin_bit_cast(
+            frag_t, keep_or_zero(q_raw[t], q_row < a.sq && 16 * t + 8 * g < a.d));
     if (2 < n_tiles) {
         ks_b.load(k_base, a.ks[1], (t_lo + 2) * kBN, a.sk, a.d);
         vs_b.load(v_base, a.vs[1], (t_lo + 2) * kBN, a.sk, a.d);

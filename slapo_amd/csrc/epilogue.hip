@@ -82,9 +82,16 @@ __device__ __forceinline__ void store_chunk(T* p, const Chunk<T, V>& c) {
 }
 
 // Keep-bits for V consecutive elements starting at element index e0 (e0 % V == 0).
-template <int V>
+// kDrop: 1 = shift-only mask geometry (vec >= 4, power-of-two thread count), 2 = any geometry.
+template <int V, int kDrop>
 __device__ __forceinline__ uint32_t keep_bits(const DropoutState& s, uint64_t e0) {
     uint32_t bits = 0;
+    if constexpr (kDrop == 1) {
+        static_assert(V % 4 == 0, "the fast geometry needs whole Philox blocks per chunk");
+#pragma unroll
+        for (int g = 0; g < V / 4; ++g) bits |= dropout_keep4_pow2(s, e0 / 4 + g) << (4 * g);
+        return bits;
+    }
     if constexpr (V % 4 == 0) {
         if (s.vec >= 4) {
 #pragma unroll
@@ -136,16 +143,20 @@ __global__ __launch_bounds__(256) void bias_gelu_fwd_kernel(const T* __restrict_
     }
 }
 
-template <typename T, int V, bool kResidual, bool kDropout>
+#ifndef EPI_DROP_UNROLL
+#define EPI_DROP_UNROLL 1
+#endif
+template <typename T, int V, bool kResidual, int kDrop>
 __global__ __launch_bounds__(256) void bias_dropout_residual_fwd_kernel(
     const T* __restrict__ x, const T* __restrict__ bias, const T* __restrict__ residual,
     T* __restrict__ out, uint64_t n_chunks, uint32_t chunks_per_row, uint32_t row_mask,
     DropoutState s) {
-    const uint64_t base = (uint64_t)blockIdx.x * (256 * kUnroll) + threadIdx.x;
-    Chunk<T, V> in[kUnroll];
-    Chunk<T, V> res[kUnroll];
+    constexpr int kDU = EPI_DROP_UNROLL;
+    const uint64_t base = (uint64_t)blockIdx.x * (256 * kDU) + threadIdx.x;
+    Chunk<T, V> in[kDU];
+    Chunk<T, V> res[kDU];
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
+    for (int u = 0; u < kDU; ++u) {
         const uint64_t c = base + (uint64_t)u * 256;
         if (c < n_chunks) {
             in[u] = load_chunk<T, V>(x + c * V);
@@ -153,19 +164,19 @@ __global__ __launch_bounds__(256) void bias_dropout_residual_fwd_kernel(
         }
     }
 #pragma unroll
-    for (int u = 0; u < kUnroll; ++u) {
+    for (int u = 0; u < kDU; ++u) {
         const uint64_t c = base + (uint64_t)u * 256;
         if (c >= n_chunks) continue;
         const uint32_t col =
             row_mask ? ((uint32_t)c & row_mask) : (uint32_t)(c % chunks_per_row);
         const Chunk<T, V> b = load_chunk_cached<T, V>(bias + (uint64_t)col * V);
         uint32_t bits = 0xFFFFFFFFu;
-        if constexpr (kDropout) bits = keep_bits<V>(s, c * V);
+        if constexpr (kDrop != 0) bits = keep_bits<V, kDrop>(s, c * V);
         Chunk<T, V> o;
 #pragma unroll
         for (int i = 0; i < V; ++i) {
             float v = Elem<T>::to_f32(in[u].v[i]) + Elem<T>::to_f32(b.v[i]);
-            if constexpr (kDropout) v = ((bits >> i) & 1u) ? v * s.inv_keep : 0.0f;
+            if constexpr (kDrop != 0) v = ((bits >> i) & 1u) ? v * s.inv_keep : 0.0f;
             if constexpr (kResidual) v += Elem<T>::to_f32(res[u].v[i]);
             o.v[i] = Elem<T>::from_f32(v);
         }
@@ -251,7 +262,7 @@ __global__ __launch_bounds__(256) void bias_gelu_bwd_kernel(const T* __restrict_
                       });
 }
 
-template <typename T, int V, bool kDropout>
+template <typename T, int V, int kDrop>
 __global__ __launch_bounds__(256) void bias_dropout_bwd_kernel(const T* __restrict__ grad,
                                                                T* __restrict__ dx,
                                                                float* __restrict__ partial,
@@ -263,12 +274,12 @@ __global__ __launch_bounds__(256) void bias_dropout_bwd_kernel(const T* __restri
                           const int64_t off = r * cols + col0;
                           const Chunk<T, V> g = load_chunk<T, V>(grad + off);
                           uint32_t bits = 0xFFFFFFFFu;
-                          if constexpr (kDropout) bits = keep_bits<V>(s, (uint64_t)off);
+                          if constexpr (kDrop != 0) bits = keep_bits<V, kDrop>(s, (uint64_t)off);
                           Chunk<T, V> o;
 #pragma unroll
                           for (int i = 0; i < V; ++i) {
                               float d = Elem<T>::to_f32(g.v[i]);
-                              if constexpr (kDropout)
+                              if constexpr (kDrop != 0)
                                   d = ((bits >> i) & 1u) ? d * s.inv_keep : 0.0f;
                               o.v[i] = Elem<T>::from_f32(d);
                               acc[i] += d;
@@ -316,14 +327,14 @@ struct RowGeom {
     unsigned blocks;
 };
 
-inline bool flat_geom(int64_t rows, int64_t cols, int v, RowGeom* g) {
+inline bool flat_geom(int64_t rows, int64_t cols, int v, RowGeom* g, int unroll = kUnroll) {
     const int64_t cpr = cols / v;
     if (cpr > 0x7FFFFFFF) return false;
     g->chunks_per_row = (uint32_t)cpr;
     g->n_chunks = (uint64_t)rows * (uint64_t)cpr;
     g->row_mask = (cpr & (cpr - 1)) == 0 ? (uint32_t)(cpr - 1) : 0u;
     if (cpr == 1) g->row_mask = 0;  // mask 0 means "use modulo"; modulo by 1 is fine
-    const uint64_t per_block = 256ull * kUnroll;
+    const uint64_t per_block = 256ull * (uint64_t)unroll;
     const uint64_t blocks = (g->n_chunks + per_block - 1) / per_block;
     if (blocks > 0x7FFFFFFFull) return false;
     g->blocks = (unsigned)blocks;
@@ -362,21 +373,25 @@ int dropres_fwd_launch(const void* x, const void* bias, const void* residual, vo
                        int64_t rows, int64_t cols, bool dropout, const DropoutState& s,
                        hipStream_t st) {
     RowGeom g;
-    if (!flat_geom(rows, cols, V, &g)) return SLAPO_ERR_SHAPE;
+    if (!flat_geom(rows, cols, V, &g, EPI_DROP_UNROLL)) return SLAPO_ERR_SHAPE;
 #define SLAPO_LAUNCH_DR(RES, DROP)                                                             \
     hipLaunchKernelGGL((bias_dropout_residual_fwd_kernel<T, V, RES, DROP>), dim3(g.blocks),    \
                        dim3(256), 0, st, (const T*)x, (const T*)bias, (const T*)residual,      \
                        (T*)out, g.n_chunks, g.chunks_per_row, g.row_mask, s)
+    // dropout mode: the shift-only geometry needs whole Philox blocks per chunk
+    const int mode = !dropout ? 0 : (V % 4 == 0 && s.g_shift >= 0 && s.t_shift >= 0) ? 1 : 2;
     if (residual) {
-        if (dropout)
-            SLAPO_LAUNCH_DR(true, true);
-        else
-            SLAPO_LAUNCH_DR(true, false);
+        if (mode == 0) SLAPO_LAUNCH_DR(true, 0);
+        if constexpr (V % 4 == 0) {
+            if (mode == 1) SLAPO_LAUNCH_DR(true, 1);
+        }
+        if (mode == 2) SLAPO_LAUNCH_DR(true, 2);
     } else {
-        if (dropout)
-            SLAPO_LAUNCH_DR(false, true);
-        else
-            SLAPO_LAUNCH_DR(false, false);
+        if (mode == 0) SLAPO_LAUNCH_DR(false, 0);
+        if constexpr (V % 4 == 0) {
+            if (mode == 1) SLAPO_LAUNCH_DR(false, 1);
+        }
+        if (mode == 2) SLAPO_LAUNCH_DR(false, 2);
     }
 #undef SLAPO_LAUNCH_DR
     return check_launch();
@@ -426,12 +441,16 @@ int dropres_bwd_launch(const void* grad, void* dx, void* ws, int64_t rows, int64
     dim3 grid;
     if (!bwd_grid(rows, cols, V, &grid)) return SLAPO_ERR_SHAPE;
     const int write_dx = dx ? 1 : 0;
-    if (dropout)
-        hipLaunchKernelGGL((bias_dropout_bwd_kernel<T, V, true>), grid, dim3(256), 0, st,
-                           (const T*)grad, (T*)dx, (float*)ws, rows, cols, want, write_dx, s);
-    else
-        hipLaunchKernelGGL((bias_dropout_bwd_kernel<T, V, false>), grid, dim3(256), 0, st,
-                           (const T*)grad, (T*)dx, (float*)ws, rows, cols, want, write_dx, s);
+#define SLAPO_LAUNCH_DB(MODE)                                                                  \
+    hipLaunchKernelGGL((bias_dropout_bwd_kernel<T, V, MODE>), grid, dim3(256), 0, st,          \
+                       (const T*)grad, (T*)dx, (float*)ws, rows, cols, want, write_dx, s)
+    const int mode = !dropout ? 0 : (V % 4 == 0 && s.g_shift >= 0 && s.t_shift >= 0) ? 1 : 2;
+    if (mode == 0) SLAPO_LAUNCH_DB(0);
+    if constexpr (V % 4 == 0) {
+        if (mode == 1) SLAPO_LAUNCH_DB(1);
+    }
+    if (mode == 2) SLAPO_LAUNCH_DB(2);
+#undef SLAPO_LAUNCH_DB
     return check_launch();
 }
 
