@@ -93,21 +93,18 @@ class AttentionStep:
             raise RuntimeError(f"slapo_amd_attn_bwd_stages failed with status {rc}")
 
     def step(self, ev=None):
-        """ev: five events recorded around forward | prepare | dK/dV | dQ."""
+        """ev: four events recorded around forward | dQ (+ delta) | dK/dV."""
         if ev is not None:
             ev[0].record()
         self.forward()
         if ev is not None:
             ev[1].record()
-        self.backward(self._lib_mod.BWD_PREPARE)
+        self.backward(self._lib_mod.BWD_PREPARE | self._lib_mod.BWD_DQ)
         if ev is not None:
             ev[2].record()
         self.backward(self._lib_mod.BWD_DKDV)
         if ev is not None:
             ev[3].record()
-        self.backward(self._lib_mod.BWD_DQ)
-        if ev is not None:
-            ev[4].record()
 
 
 def bench_epilogues(device, iters=40):
@@ -241,7 +238,7 @@ def main():
     for _ in range(args.warmup):
         step.step()
     torch.cuda.synchronize()
-    events = [[torch.cuda.Event(enable_timing=True) for _ in range(5)]
+    events = [[torch.cuda.Event(enable_timing=True) for _ in range(4)]
               for _ in range(args.steps)]
     t0 = time.perf_counter()
     for i in range(args.steps):
@@ -253,7 +250,7 @@ def main():
     d = cfg["head_dim"]
     ms_per_step = elapsed / args.steps * 1e3
     value = 14 * d * n_pairs / (elapsed / args.steps) / 1e12
-    seg_ms = [sum(ev[i].elapsed_time(ev[i + 1]) for ev in events) / args.steps for i in range(4)]
+    seg_ms = [sum(ev[i].elapsed_time(ev[i + 1]) for ev in events) / args.steps for i in range(3)]
     kern_ms = seg_ms[2]
     bwd_flops = 8 * d * n_pairs
     achieved = bwd_flops / (kern_ms * 1e-3) / 1e12
@@ -288,8 +285,7 @@ def main():
     }
     result["kernels"] = [kern("attn_fwd_kernel<f16, 64, false, 0>", 4 * d * n_pairs, seg_ms[0]),
                          kern("attn_bwd_kernel<f16, 64, false, 0> (dK/dV)", bwd_flops, seg_ms[2]),
-                         kern("attn_bwd_dq_kernel<f16, 64, false, 0>", 6 * d * n_pairs, seg_ms[3])]
-    result["delta_kernel_ms"] = seg_ms[1]
+                         kern("attn_bwd_dq_kernel<f16, 64, false, 0>", 6 * d * n_pairs, seg_ms[1])]
     if not args.no_epilogues:
         result["epilogue"] = bench_epilogues(device)
     if not args.no_cpu_baseline:

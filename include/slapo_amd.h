@@ -175,15 +175,17 @@ int slapo_amd_attn_bwd(const slapo_attn_params* prm, const void* q, const void* 
                        const int64_t dk_strides[3], const int64_t dv_strides[3], void* workspace,
                        size_t workspace_bytes, void* stream);
 
-/* The backward runs as three stages on `stream`: PREPARE (delta = rowsum(dO * O) into the
- * workspace), DKDV (workgroups own key rows and write dk, dv) and DQ (workgroups own query rows
- * and write dq).  DKDV and DQ both recompute the probabilities from lse, depend only on PREPARE
- * and write disjoint outputs: no atomics, no zero-initialised accumulator, bitwise reproducible.
- * slapo_amd_attn_bwd runs all three; this entry point runs the stages named in `stages` (a bit-or
- * of the constants below) so that a caller can time one of them or put DKDV and DQ on different
- * streams.  Arguments are those of slapo_amd_attn_bwd and must be the same across the calls of one
- * backward pass.  For SLAPO_F32 both gradient stages are served by the FMA kernels (DKDV runs
- * them all, DQ is a no-op). */
+/* The backward runs as stages on `stream`, in this order:
+ *   PREPARE  SLAPO_F32 only: delta = rowsum(dO * O) into the workspace (a no-op for 16-bit types);
+ *   DQ       workgroups own query rows and write dq; for 16-bit types this stage also computes
+ *            delta for its rows and stores it in the workspace;
+ *   DKDV     workgroups own key rows and write dk, dv; reads delta from the workspace.
+ * DQ and DKDV both recompute the probabilities from lse and write disjoint outputs: no atomics,
+ * no zero-initialised accumulator, bitwise reproducible.  slapo_amd_attn_bwd runs all stages;
+ * this entry point runs the stages named in `stages` (a bit-or of the constants below, executed
+ * in the order above) so that a caller can time one of them.  Arguments are those of
+ * slapo_amd_attn_bwd and must be the same across the calls of one backward pass.  For SLAPO_F32
+ * both gradient stages are served by the FMA kernels (DKDV runs them all, DQ is a no-op). */
 #define SLAPO_BWD_PREPARE 1
 #define SLAPO_BWD_DKDV 2
 #define SLAPO_BWD_DQ 4

@@ -2,7 +2,9 @@
 //
 // The backward is split in two kernels that each recompute the probabilities: this one owns query
 // rows and produces dQ, its sibling owns key rows and produces dK / dV.  Neither needs atomics or
-// a zero-initialised accumulator, and the result does not depend on scheduling order.
+// a zero-initialised accumulator, and the result does not depend on scheduling order.  This kernel
+// also produces delta = rowsum(dO * O) for its query rows (it holds the dO fragments anyway) and
+// stores it for the dK / dV kernel, which therefore has to run after it.
 //
 // One workgroup (4 wavefronts) owns 128 consecutive queries of one (batch, head); wavefront w
 // owns 32 of them and keeps their Q^T and dO^T fragments, lse and delta in registers.  Keys and
@@ -60,7 +62,7 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_dq_ke
     const int wq0 = q0 + wave * 32;
     const int q_row = wq0 + i_loc;
 #ifdef EXP_TIMING_DQ
-    unsigned long long* tbuf = reinterpret_cast<unsigned long long*>(a.o) + 512;
+    unsigned long long* tbuf = reinterpret_cast<unsigned long long*>(a.dk) + 512;
     int tcount = 0;
     const bool trec = (blockIdx.x == EXP_TIMING_DQ) && threadIdx.x == 0;
 #define TSTAMP_DQ() do { if (trec) tbuf[tcount++] = __builtin_readcyclecounter(); } while (0)
@@ -88,15 +90,16 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_dq_ke
     float lse2, delta;
     {
         const int qr = min(q_row, a.sq - 1);
-        u32x4_t qv[DK], gv[DK];
+        const T* o_base = reinterpret_cast<const T*>(a.o) + b * a.os[0] + h * a.os[2];
+        u32x4_t qv[DK], gv[DK], ov[DK];
 #pragma unroll
         for (int t = 0; t < DK; ++t) {
             const int dc = min(16 * t + 8 * g, a.d - 8);
             qv[t] = *reinterpret_cast<const u32x4_t*>(q_base + (int64_t)qr * a.qs[1] + dc);
             gv[t] = *reinterpret_cast<const u32x4_t*>(g_base + (int64_t)qr * a.os[1] + dc);
+            ov[t] = *reinterpret_cast<const u32x4_t*>(o_base + (int64_t)qr * a.os[1] + dc);
         }
         const float lse_raw = a.lse[(int64_t)bh * a.sq + qr];
-        const float delta_raw = a.delta[(int64_t)bh * a.sq + qr];
         ks.load(k_base, a.ks[1], t_lo * kBN, a.sk, a.d);
         vs.load(v_base, a.vs[1], t_lo * kBN, a.sk, a.d);
         const bool row_ok = q_row < a.sq;
@@ -108,7 +111,17 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_dq_ke
         }
         // log2 units; +inf for rows past the end so that P = 0 there
         lse2 = row_ok ? lse_raw * kLog2e : INFINITY;
-        delta = row_ok ? delta_raw : 0.f;
+        // delta = sum_d dO * O: lanes i and i + 32 hold complementary head-dim slots of row i
+        float part = 0.f;
+#pragma unroll
+        for (int t = 0; t < DK; ++t) {
+            const frag_t of = __builtin_bit_cast(frag_t, ov[t]);
+#pragma unroll
+            for (int j = 0; j < 8; ++j)
+                part = __builtin_fmaf((float)gf[t][j], (float)of[j], part);
+        }
+        delta = sum_xor32(part);  // masked dO slots are zero, so clamped rows / columns add nothing
+        if (row_ok && g == 0) a.delta[(int64_t)bh * a.sq + q_row] = delta;
     }
 
     f32x16_t dq_acc[DV];
@@ -350,11 +363,7 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_dq_ke
         const T* kt = k_lds + (r % kKRing) * kTileElems;
         const T* vt = v_lds + (r % kVRing) * kTileElems;
         if constexpr (kFast) {
-#ifdef EXP_NO_HANDSCHED
-            tile_body(kt, vt, t, std::integral_constant<int, 0>{});
-#else
             tile_body_fast(kt, vt, t);
-#endif
         } else if (tile_active(t)) {
             if (!tile_needs_mask(t))
                 tile_body(kt, vt, t, std::integral_constant<int, 0>{});

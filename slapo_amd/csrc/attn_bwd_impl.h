@@ -30,8 +30,7 @@ namespace bwd {
 
 constexpr int kBwdWaves = 4;
 constexpr int kBwdThreads = kBwdWaves * 64;
-constexpr int kBwdBN = kBwdWaves * 32;  // keys per workgroup
-constexpr int kBwdBM = 64;              // queries per tile
+constexpr int kBwdBM = 64;  // queries per tile
 
 template <typename T, int DPAD>
 struct BwdSmem {
@@ -43,8 +42,11 @@ struct BwdSmem {
     static constexpr size_t kBytes = 2 * kQBytes + kStatBytes;
 };
 
-template <typename T, int DPAD, bool kBias, int kDrop>
-__global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_kernel(
+// KB = blocks of 32 keys per wavefront.  KB = 2 halves the LDS operand traffic per matrix
+// instruction (every Q / dO fragment read feeds two MFMAs) at the price of twice the resident
+// fragments and accumulators, i.e. one wavefront per SIMD instead of two.
+template <typename T, int DPAD, bool kBias, int kDrop, int KB>
+__global__ __launch_bounds__(kBwdThreads, ((DPAD <= 64 && KB == 1) ? 2 : 1)) void attn_bwd_kernel(
     const AttnArgs a) {
     typedef typename Mma<T>::frag frag_t;
     typedef BwdSmem<T, DPAD> SM;
@@ -52,6 +54,8 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
     constexpr int kPitch = SM::kPitch;
     constexpr int DK = DPAD / 16;          // k-steps over head dim
     constexpr int DV = DPAD / 32;          // 32-row blocks of dK^T / dV^T
+    constexpr int kWaveKeys = 32 * KB;
+    constexpr int kBN = kBwdWaves * kWaveKeys;  // keys per workgroup
 
     extern __shared__ __align__(16) unsigned char smem_raw[];
     T* q_lds = reinterpret_cast<T*>(smem_raw);
@@ -63,7 +67,7 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
     const int kt = blockIdx.x / n_bh;  // low key tiles see the most queries under a causal mask
     const int b = bh / a.heads;
     const int h = bh % a.heads;
-    const int k0 = kt * kBwdBN;
+    const int k0 = kt * kBN;
 
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wavefront-uniform
@@ -74,15 +78,14 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
     int tcount = 0;
     const bool trec = (blockIdx.x == EXP_TIMING) && threadIdx.x == 0;
 #define TSTAMP() do { if (trec) tbuf[tcount++] = __builtin_readcyclecounter(); } while (0)
-// stamp taken only after `dep` has been produced (forces the wait for the MFMA / VALU results)
-#define TSTAMP2(dep) do { float dd = (dep); asm volatile("" :: "v"(dd)); if (trec) tbuf[tcount++] = __builtin_readcyclecounter(); } while (0)
     TSTAMP();
 #else
 #define TSTAMP() do {} while (0)
-#define TSTAMP2(dep) do {} while (0)
 #endif
-    const int kw0 = k0 + wave * 32;
-    const int key = kw0 + c_loc;  // this lane's key column
+    const int kw0 = k0 + wave * kWaveKeys;  // first key of this wavefront
+    int key[KB];                            // this lane's key column in each block
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb) key[kb] = kw0 + 32 * kb + c_loc;
 
     const T* q_base = reinterpret_cast<const T*>(a.q) + b * a.qs[0] + h * a.qs[2];
     const T* k_base = reinterpret_cast<const T*>(a.k) + b * a.ks[0] + h * a.ks[2];
@@ -94,35 +97,43 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
     // ---- resident fragments ----
     // Loaded with clamped addresses and masked once the first query tile has been requested too,
     // so that all start-up loads of the workgroup are in flight together.
-    frag_t kf[DK], vf[DK];
-    u32x4_t k_raw[DK], v_raw[DK];
-    {
-        const int kr = min(key, a.sk - 1);
+    frag_t kf[KB][DK], vf[KB][DK];
+    u32x4_t k_raw[KB][DK], v_raw[KB][DK];
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb) {
+        const int kr = min(key[kb], a.sk - 1);
 #pragma unroll
         for (int t = 0; t < DK; ++t) {
             const int dc = min(16 * t + 8 * g, a.d - 8);
-            k_raw[t] = *reinterpret_cast<const u32x4_t*>(k_base + (int64_t)kr * a.ks[1] + dc);
-            v_raw[t] = *reinterpret_cast<const u32x4_t*>(v_base + (int64_t)kr * a.vs[1] + dc);
+            k_raw[kb][t] = *reinterpret_cast<const u32x4_t*>(k_base + (int64_t)kr * a.ks[1] + dc);
+            v_raw[kb][t] = *reinterpret_cast<const u32x4_t*>(v_base + (int64_t)kr * a.vs[1] + dc);
         }
     }
 
-    f32x16_t dk_acc[DV], dv_acc[DV];
+    f32x16_t dk_acc[KB][DV], dv_acc[KB][DV];
 #pragma unroll
-    for (int x = 0; x < DV; ++x)
+    for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) dk_acc[x][r] = 0.f, dv_acc[x][r] = 0.f;
+        for (int x = 0; x < DV; ++x)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) dk_acc[kb][x][r] = 0.f, dv_acc[kb][x][r] = 0.f;
 
     int i_lo, i_hi;
-    query_range(a, k0, min(k0 + kBwdBN, a.sk), i_lo, i_hi);
+    query_range(a, k0, min(k0 + kBN, a.sk), i_lo, i_hi);
     const int t_lo = i_lo / kBwdBM;
     const int t_hi = (i_hi + kBwdBM - 1) / kBwdBM;
 
     // Per-lane bias when it does not depend on the query (the compact [B,1,1,Sk] layout).
     const bool bias_per_key = kBias && a.bs[2] == 0;
-    float bias_k = 0.f;
-    if constexpr (kBias) {
-        if (bias_per_key && key < a.sk)
-            bias_k = a.bias[b * a.bs[0] + h * a.bs[1] + (int64_t)key * a.bs[3]] * kLog2e;
+    float bias_k[KB];
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb) {
+        bias_k[kb] = 0.f;
+        if constexpr (kBias) {
+            if (bias_per_key && key[kb] < a.sk)
+                bias_k[kb] =
+                    a.bias[b * a.bs[0] + h * a.bs[1] + (int64_t)key[kb] * a.bs[3]] * kLog2e;
+        }
     }
     const float c_log2 = a.scale_log2;
 
@@ -154,11 +165,13 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
     gst.load(g_base, a.os[1], t_lo * kBwdBM, a.sq, a.d);
     load_stats(t_lo * kBwdBM);
 #pragma unroll
-    for (int t = 0; t < DK; ++t) {
-        const bool keep = key < a.sk && 16 * t + 8 * g < a.d;
-        kf[t] = __builtin_bit_cast(frag_t, keep_or_zero(k_raw[t], keep));
-        vf[t] = __builtin_bit_cast(frag_t, keep_or_zero(v_raw[t], keep));
-    }
+    for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+        for (int t = 0; t < DK; ++t) {
+            const bool keep = key[kb] < a.sk && 16 * t + 8 * g < a.d;
+            kf[kb][t] = __builtin_bit_cast(frag_t, keep_or_zero(k_raw[kb][t], keep));
+            vf[kb][t] = __builtin_bit_cast(frag_t, keep_or_zero(v_raw[kb][t], keep));
+        }
     if (t_lo < t_hi) {
         qst.fix(t_lo * kBwdBM, a.sq, a.d);
         gst.fix(t_lo * kBwdBM, a.sq, a.d);
@@ -173,73 +186,83 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
         const int i_last = min(ih0 + 32, a.sq) - 1;
         if (kw0 >= a.sk || ih0 >= a.sq) return false;
         if (a.causal && kw0 > i_last) return false;
-        if (a.window > 0 && ih0 - (kw0 + 31) >= a.window) return false;
+        if (a.window > 0 && ih0 - (kw0 + kWaveKeys - 1) >= a.window) return false;
         return true;
     };
     auto half_needs_mask = [&](int ih0) __attribute__((always_inline)) {
         const int i_last = min(ih0 + 32, a.sq) - 1;
-        return (kw0 + 32 > a.sk) || (a.causal && kw0 + 31 > ih0) ||
+        return (kw0 + kWaveKeys > a.sk) || (a.causal && kw0 + kWaveKeys - 1 > ih0) ||
                (a.window > 0 && i_last - kw0 >= a.window);
     };
 
     // ---- stages of one half tile (32 queries at ih0 = i0 + 32 hf) ----
-    // S = Q_h K_w^T, dP = dO_h V_w^T
-    auto half_sp = [&](const T* qt, const T* gt, int hf, f32x16_t& s, f32x16_t& dp)
+    // S = Q_h K_w^T, dP = dO_h V_w^T: every Q / dO fragment read feeds KB matrix instructions
+    auto half_sp = [&](const T* qt, const T* gt, int hf, f32x16_t (&s)[KB], f32x16_t (&dp)[KB])
                        __attribute__((always_inline)) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) s[r] = 0.f, dp[r] = 0.f;
+        for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s[kb][r] = 0.f, dp[kb][r] = 0.f;
         const T* qrow = qt + 32 * hf * kPitch + a_off;
         const T* grow = gt + 32 * hf * kPitch + a_off;
 #pragma unroll
         for (int x = 0; x < DK; ++x) {
-            s = Mma<T>::mma32(lds_frag<T>(qrow + 16 * x), kf[x], s);
-            dp = Mma<T>::mma32(lds_frag<T>(grow + 16 * x), vf[x], dp);
+            const frag_t qa = lds_frag<T>(qrow + 16 * x);
+            const frag_t ga = lds_frag<T>(grow + 16 * x);
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) {
+                s[kb] = Mma<T>::mma32(qa, kf[kb][x], s[kb]);
+                dp[kb] = Mma<T>::mma32(ga, vf[kb][x], dp[kb]);
+            }
         }
     };
     // scores -> probabilities in place.  mask_tag: 0 = all visible, 1 = lower bound on the query
     // only (causal / key tail), 2 = both bounds (local window)
-    auto half_exp = [&](f32x16_t& s, const float* lse_h, int ih0, auto mask_tag)
+    auto half_exp = [&](f32x16_t (&s)[KB], const float* lse_h, int ih0, auto mask_tag)
                         __attribute__((always_inline)) {
         constexpr int kMask = decltype(mask_tag)::value;
         // register r is query ih0 + 8 g + c with c = acc_row(r, 0); visible iff c_lo <= c <= c_hi
-        int c_lo = 0, c_hi = 0;
-        if constexpr (kMask != 0) {
-            c_lo = (key < a.sk) ? (a.causal ? key - ih0 - 8 * g : -1) : 64;
-            if constexpr (kMask == 2) c_hi = key + a.window - 1 - ih0 - 8 * g;
+        int c_lo[KB], c_hi[KB];
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb) {
+            c_lo[kb] = 0, c_hi[kb] = 0;
+            if constexpr (kMask != 0) {
+                c_lo[kb] = (key[kb] < a.sk) ? (a.causal ? key[kb] - ih0 - 8 * g : -1) : 64;
+                if constexpr (kMask == 2) c_hi[kb] = key[kb] + a.window - 1 - ih0 - 8 * g;
+            }
         }
 #pragma unroll
         for (int r4 = 0; r4 < 4; ++r4) {
             const int qoff = acc_row(4 * r4, g);
             const f32x4_t lse4 = *reinterpret_cast<const f32x4_t*>(lse_h + qoff);
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                float x = __builtin_fmaf(s[4 * r4 + e], c_log2, -lse4[e]);
-                if constexpr (kBias) {
-                    const int i = ih0 + qoff + e;
-                    if (bias_per_key)
-                        x += bias_k;
-                    else if (i < a.sq && key < a.sk)
-                        x += a.bias[b * a.bs[0] + h * a.bs[1] + (int64_t)i * a.bs[2] +
-                                    (int64_t)key * a.bs[3]] * kLog2e;
-                }
-                float p = fast_exp2(x);
-                if constexpr (kMask != 0) {
-                    const int c = acc_row(4 * r4, 0) + e;
-                    if constexpr (kMask == 2) {
-                        if (c < c_lo || c > c_hi) p = 0.f;
-                    } else {
-                        if (c < c_lo) p = 0.f;
+            for (int kb = 0; kb < KB; ++kb)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    float x = __builtin_fmaf(s[kb][4 * r4 + e], c_log2, -lse4[e]);
+                    if constexpr (kBias) {
+                        const int i = ih0 + qoff + e;
+                        if (bias_per_key)
+                            x += bias_k[kb];
+                        else if (i < a.sq && key[kb] < a.sk)
+                            x += a.bias[b * a.bs[0] + h * a.bs[1] + (int64_t)i * a.bs[2] +
+                                        (int64_t)key[kb] * a.bs[3]] * kLog2e;
                     }
+                    float p = fast_exp2(x);
+                    if constexpr (kMask != 0) {
+                        const int c = acc_row(4 * r4, 0) + e;
+                        if constexpr (kMask == 2) {
+                            if (c < c_lo[kb] || c > c_hi[kb]) p = 0.f;
+                        } else {
+                            if (c < c_lo[kb]) p = 0.f;
+                        }
+                    }
+                    s[kb][4 * r4 + e] = p;
                 }
-                s[4 * r4 + e] = p;
-            }
         }
     };
-    // P (after dropout) and dS = P (dP - delta), packed to T
-    auto half_ds = [&](const f32x16_t& p, const f32x16_t& dp, const float* delta_h, int ih0,
-                       uint32_t (&pw)[8], uint32_t (&dw)[8]) __attribute__((always_inline)) {
-        // Keep-bits of this half: wq[e] bit 4 * r4 belongs to register 4 * r4 + e.
-        uint32_t wq[4] = {0u, 0u, 0u, 0u};
+    // Keep-bits of one key block of a half tile: wq[e] bit 4 * r4 belongs to register 4 * r4 + e.
+    auto keep_bits_half = [&](int kcol, int ih0, uint32_t (&wq)[4]) __attribute__((always_inline)) {
         if constexpr (kDrop == 1) {
             // The four lanes of a quad hold four consecutive keys, i.e. one Philox block per query
             // row.  Lane j of the quad draws the blocks of the rows held in registers j, j+4, j+8,
@@ -249,9 +272,9 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
 #pragma unroll
             for (int r4 = 0; r4 < 4; ++r4) {
                 const int i = ih0 + acc_row(4 * r4, g) + qpos;
-                if (i < a.sq && key < a.sk) {
+                if (i < a.sq && kcol < a.sk) {
                     const uint64_t el =
-                        ((uint64_t)bh * a.sq + (uint64_t)i) * (uint64_t)a.sk + (uint64_t)(key & ~3);
+                        ((uint64_t)bh * a.sq + (uint64_t)i) * (uint64_t)a.sk + (uint64_t)(kcol & ~3);
                     mine |= dropout_keep4_pow2(a.rng, el >> 2) << (4 * r4);
                 }
             }
@@ -264,53 +287,79 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
 #pragma unroll 1
             for (int r = 0; r < 16; ++r) {
                 const int i = ih0 + acc_row(r, g);
-                if (i < a.sq && key < a.sk) {
+                if (i < a.sq && kcol < a.sk) {
                     const uint64_t el =
-                        ((uint64_t)bh * a.sq + (uint64_t)i) * (uint64_t)a.sk + (uint64_t)key;
+                        ((uint64_t)bh * a.sq + (uint64_t)i) * (uint64_t)a.sk + (uint64_t)kcol;
                     if (dropout_keep1(a.rng, el)) mask16 |= 1u << r;
                 }
             }
 #pragma unroll
             for (int e = 0; e < 4; ++e) wq[e] = mask16 >> e;
         }
+    };
+    // P (after dropout) and dS = P (dP - delta), packed to T
+    auto half_ds = [&](const f32x16_t (&p)[KB], const f32x16_t (&dp)[KB], const float* delta_h,
+                       int ih0, uint32_t (&pw)[KB][8], uint32_t (&dw)[KB][8])
+                       __attribute__((always_inline)) {
+        uint32_t wq[KB][4];
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) wq[kb][e] = 0u;
+            keep_bits_half(key[kb], ih0, wq[kb]);
+        }
 #pragma unroll
         for (int r4 = 0; r4 < 4; ++r4) {
             const int qoff = acc_row(4 * r4, g);
             const f32x4_t del4 = *reinterpret_cast<const f32x4_t*>(delta_h + qoff);
-            float pv[4], dv[4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                float pe = p[4 * r4 + e];
-                float d = dp[4 * r4 + e];
-                float pd = pe;
-                if constexpr (kDrop != 0) {
-                    const float keep = ((wq[e] >> (4 * r4)) & 1u) ? a.rng.inv_keep : 0.f;
-                    pd = pe * keep;
-                    d = d * keep;
+            for (int kb = 0; kb < KB; ++kb) {
+                float pv[4], dv[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    float pe = p[kb][4 * r4 + e];
+                    float d = dp[kb][4 * r4 + e];
+                    float pd = pe;
+                    if constexpr (kDrop != 0) {
+                        const float keep = ((wq[kb][e] >> (4 * r4)) & 1u) ? a.rng.inv_keep : 0.f;
+                        pd = pe * keep;
+                        d = d * keep;
+                    }
+                    pv[e] = pd;
+                    dv[e] = pe * (d - del4[e]);
                 }
-                pv[e] = pd;
-                dv[e] = pe * (d - del4[e]);
+                pw[kb][2 * r4] = pack2<T>(pv[0], pv[1]);
+                pw[kb][2 * r4 + 1] = pack2<T>(pv[2], pv[3]);
+                dw[kb][2 * r4] = pack2<T>(dv[0], dv[1]);
+                dw[kb][2 * r4 + 1] = pack2<T>(dv[2], dv[3]);
             }
-            pw[2 * r4] = pack2<T>(pv[0], pv[1]);
-            pw[2 * r4 + 1] = pack2<T>(pv[2], pv[3]);
-            dw[2 * r4] = pack2<T>(dv[0], dv[1]);
-            dw[2 * r4 + 1] = pack2<T>(dv[2], dv[3]);
         }
     };
-    // dV^T += dO_h^T P, dK^T += Q_h^T dS
-    auto half_out = [&](const T* qt, const T* gt, int hf, const uint32_t (&pw)[8],
-                        const uint32_t (&dw)[8]) __attribute__((always_inline)) {
+    // dV^T += dO_h^T P, dK^T += Q_h^T dS: every transposed fragment read feeds KB instructions
+    auto half_out = [&](const T* qt, const T* gt, int hf, const uint32_t (&pw)[KB][8],
+                        const uint32_t (&dw)[KB][8]) __attribute__((always_inline)) {
 #pragma unroll
         for (int hh = 0; hh < 2; ++hh) {
-            u32x4_t pq = {pw[4 * hh], pw[4 * hh + 1], pw[4 * hh + 2], pw[4 * hh + 3]};
-            u32x4_t dq4 = {dw[4 * hh], dw[4 * hh + 1], dw[4 * hh + 2], dw[4 * hh + 3]};
-            const frag_t pf = __builtin_bit_cast(frag_t, pq);
-            const frag_t df = __builtin_bit_cast(frag_t, dq4);
+            frag_t pf[KB], df[KB];
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) {
+                u32x4_t pq = {pw[kb][4 * hh], pw[kb][4 * hh + 1], pw[kb][4 * hh + 2],
+                              pw[kb][4 * hh + 3]};
+                u32x4_t dq4 = {dw[kb][4 * hh], dw[kb][4 * hh + 1], dw[kb][4 * hh + 2],
+                               dw[kb][4 * hh + 3]};
+                pf[kb] = __builtin_bit_cast(frag_t, pq);
+                df[kb] = __builtin_bit_cast(frag_t, dq4);
+            }
             const int off = (32 * hf + 16 * hh) * kPitch + t_off;
 #pragma unroll
             for (int x = 0; x < DV; ++x) {
-                dv_acc[x] = Mma<T>::mma32(lds_frag_tr<T>(gt + off + 32 * x, kPitch), pf, dv_acc[x]);
-                dk_acc[x] = Mma<T>::mma32(lds_frag_tr<T>(qt + off + 32 * x, kPitch), df, dk_acc[x]);
+                const frag_t gta = lds_frag_tr<T>(gt + off + 32 * x, kPitch);
+                const frag_t qta = lds_frag_tr<T>(qt + off + 32 * x, kPitch);
+#pragma unroll
+                for (int kb = 0; kb < KB; ++kb) {
+                    dv_acc[kb][x] = Mma<T>::mma32(gta, pf[kb], dv_acc[kb][x]);
+                    dk_acc[kb][x] = Mma<T>::mma32(qta, df[kb], dk_acc[kb][x]);
+                }
             }
         }
     };
@@ -335,8 +384,8 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
         }
         if constexpr (kFast) {
             std::integral_constant<int, 0> none;
-            f32x16_t s0, s1, p0, p1;
-            uint32_t pw0[8], dw0[8], pw1[8], dw1[8];
+            f32x16_t s0[KB], s1[KB], p0[KB], p1[KB];
+            uint32_t pw0[KB][8], dw0[KB][8], pw1[KB][8], dw1[KB][8];
             half_sp(qt, gt, 0, s0, p0);
             half_exp(s0, lse_t, i0, none);
             half_sp(qt, gt, 1, s1, p1);
@@ -349,8 +398,8 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
             auto generic_half = [&](int hf) __attribute__((always_inline)) {
                 const int ih0 = i0 + 32 * hf;
                 if (!half_active(ih0)) return;
-                f32x16_t s, dp;
-                uint32_t pw[8], dw[8];
+                f32x16_t s[KB], dp[KB];
+                uint32_t pw[KB][8], dw[KB][8];
                 half_sp(qt, gt, hf, s, dp);
                 if (!half_needs_mask(ih0))
                     half_exp(s, lse_t + 32 * hf, ih0, std::integral_constant<int, 0>{});
@@ -379,8 +428,8 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
     };
     auto tile_fast = [&](int t) __attribute__((always_inline)) {
         const int i0 = t * kBwdBM;
-        return a.window <= 0 && k0 + kBwdBN <= a.sk && i0 + kBwdBM <= a.sq &&
-               (!a.causal || i0 >= k0 + kBwdBN - 1);
+        return a.window <= 0 && k0 + kBN <= a.sk && i0 + kBwdBM <= a.sq &&
+               (!a.causal || i0 >= k0 + kBN - 1);
     };
     TSTAMP();
     {
@@ -392,20 +441,26 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
 
     TSTAMP();
     // ---- write dK, dV ----
-    if (key < a.sk) {
-        T* dk_row = reinterpret_cast<T*>(a.dk) + b * a.dks[0] + (int64_t)key * a.dks[1] + h * a.dks[2];
-        T* dv_row = reinterpret_cast<T*>(a.dv) + b * a.dvs[0] + (int64_t)key * a.dvs[1] + h * a.dvs[2];
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb) {
+        if (key[kb] >= a.sk) continue;
+        T* dk_row =
+            reinterpret_cast<T*>(a.dk) + b * a.dks[0] + (int64_t)key[kb] * a.dks[1] + h * a.dks[2];
+        T* dv_row =
+            reinterpret_cast<T*>(a.dv) + b * a.dvs[0] + (int64_t)key[kb] * a.dvs[1] + h * a.dvs[2];
 #pragma unroll
         for (int x = 0; x < DV; ++x)
 #pragma unroll
             for (int r4 = 0; r4 < 4; ++r4) {
                 const int d0 = x * 32 + 8 * r4 + 4 * g;
                 if (d0 < a.d) {
+                    const f32x16_t& ka = dk_acc[kb][x];
+                    const f32x16_t& va = dv_acc[kb][x];
                     u32x2_t wk, wv;
-                    wk.x = pack2<T>(dk_acc[x][4 * r4] * a.scale, dk_acc[x][4 * r4 + 1] * a.scale);
-                    wk.y = pack2<T>(dk_acc[x][4 * r4 + 2] * a.scale, dk_acc[x][4 * r4 + 3] * a.scale);
-                    wv.x = pack2<T>(dv_acc[x][4 * r4], dv_acc[x][4 * r4 + 1]);
-                    wv.y = pack2<T>(dv_acc[x][4 * r4 + 2], dv_acc[x][4 * r4 + 3]);
+                    wk.x = pack2<T>(ka[4 * r4] * a.scale, ka[4 * r4 + 1] * a.scale);
+                    wk.y = pack2<T>(ka[4 * r4 + 2] * a.scale, ka[4 * r4 + 3] * a.scale);
+                    wv.x = pack2<T>(va[4 * r4], va[4 * r4 + 1]);
+                    wv.y = pack2<T>(va[4 * r4 + 2], va[4 * r4 + 3]);
                     *reinterpret_cast<u32x2_t*>(dk_row + d0) = wk;
                     *reinterpret_cast<u32x2_t*>(dv_row + d0) = wv;
                 }
@@ -413,14 +468,15 @@ __global__ __launch_bounds__(kBwdThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_ke
     }
 }
 
-template <typename T, int DPAD, bool kBias, int kDrop>
+template <typename T, int DPAD, bool kBias, int kDrop, int KB>
 int launch(const AttnArgs& a, hipStream_t st) {
     typedef BwdSmem<T, DPAD> SM;
     const size_t smem = SM::kBytes;
-    const int n_kt = (a.sk + kBwdBN - 1) / kBwdBN;
+    constexpr int kBN = kBwdWaves * 32 * KB;
+    const int n_kt = (a.sk + kBN - 1) / kBN;
     const int64_t blocks = (int64_t)n_kt * a.batch * a.heads;
     if (blocks <= 0 || blocks > 0x7FFFFFFF) return SLAPO_ERR_SHAPE;
-    auto kern = attn_bwd_kernel<T, DPAD, kBias, kDrop>;
+    auto kern = attn_bwd_kernel<T, DPAD, kBias, kDrop, KB>;
     if (smem > 48 * 1024) {
         static bool raised = false;  // per instantiation
         if (!raised) {
@@ -431,33 +487,28 @@ int launch(const AttnArgs& a, hipStream_t st) {
             raised = true;
         }
     }
-#ifdef EXP_OCC
-    {
-        static bool once = false;
-        if (!once) {
-            once = true;
-            int nb = -1;
-            hipOccupancyMaxActiveBlocksPerMultiprocessor(&nb, reinterpret_cast<const void*>(kern), kBwdThreads, smem);
-            hipFuncAttributes fa;
-            hipFuncGetAttributes(&fa, reinterpret_cast<const void*>(kern));
-            fprintf(stderr, "[occ] %s DPAD=%d smem=%zu regs=%d staticsmem=%zu maxthreads=%d -> blocks/CU=%d\n", __func__, DPAD, smem, fa.numRegs, fa.sharedSizeBytes, fa.maxThreadsPerBlock, nb);
-        }
-    }
-#endif
     hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kBwdThreads), smem, st, a);
     return check_launch();
+}
+
+// Two key blocks per wavefront (KB = 2, one wavefront per SIMD) measured slower than KB = 1 with two
+// wavefronts per SIMD on MI355X (92 us against 70 us at fp16 B8 S1024 H16 D64 causal): the second
+// resident wavefront hides more latency than the halved LDS traffic saves.  Only KB = 1 is built.
+template <typename T, int DPAD, bool kBias, int kDrop>
+int launch_kb(const AttnArgs& a, hipStream_t st) {
+    return launch<T, DPAD, kBias, kDrop, 1>(a, st);
 }
 
 template <typename T, int DPAD>
 int dispatch_flags(const AttnArgs& a, hipStream_t st) {
     if (a.has_bias) {
-        if (a.dropout == 1) return launch<T, DPAD, true, 1>(a, st);
-        if (a.dropout == 2) return launch<T, DPAD, true, 2>(a, st);
-        return launch<T, DPAD, true, 0>(a, st);
+        if (a.dropout == 1) return launch_kb<T, DPAD, true, 1>(a, st);
+        if (a.dropout == 2) return launch_kb<T, DPAD, true, 2>(a, st);
+        return launch_kb<T, DPAD, true, 0>(a, st);
     }
-    if (a.dropout == 1) return launch<T, DPAD, false, 1>(a, st);
-    if (a.dropout == 2) return launch<T, DPAD, false, 2>(a, st);
-    return launch<T, DPAD, false, 0>(a, st);
+    if (a.dropout == 1) return launch_kb<T, DPAD, false, 1>(a, st);
+    if (a.dropout == 2) return launch_kb<T, DPAD, false, 2>(a, st);
+    return launch_kb<T, DPAD, false, 0>(a, st);
 }
 
 template <typename T>

@@ -222,26 +222,23 @@ extern "C" int slapo_amd_attn_bwd_stages(const slapo_attn_params* prm, const voi
     if (!strides_ok(dq_strides, 8) || !strides_ok(dk_strides, 8) || !strides_ok(dv_strides, 8))
         return SLAPO_ERR_ALIGN;
 
-    if (stages & SLAPO_BWD_PREPARE) {
-        const unsigned row_blocks = (unsigned)((rows * 8 + 255) / 256);
-        if (prm->dtype == SLAPO_F16)
-            hipLaunchKernelGGL((attn_delta_kernel<f16_t>), dim3(row_blocks), dim3(256), 0, st, a);
-        else
-            hipLaunchKernelGGL((attn_delta_kernel<bf16_t>), dim3(row_blocks), dim3(256), 0, st, a);
-        rc = check_launch();
-        if (rc != SLAPO_OK) return rc;
-    }
-    // dK / dV (workgroups own keys), then dQ (workgroups own queries); both read delta.
-    if (stages & SLAPO_BWD_DKDV) {
+    // 16-bit types: PREPARE has nothing to do (the dQ kernel computes delta for its own rows and
+    // stores it for the dK / dV kernel), so DQ runs before DKDV.
+    if (stages & SLAPO_BWD_DQ) {
 #if defined(EXP_TIMING) || defined(EXP_TIMING_DQ)
         if (!g_timing_buf) { hipMalloc(&g_timing_buf, 1 << 16); hipMemset(g_timing_buf, 0, 1 << 16); }
+        a.dk = g_timing_buf;
+#endif
+        rc = prm->dtype == SLAPO_F16 ? attn_bwd_dq_mfma_f16(a, st) : attn_bwd_dq_mfma_bf16(a, st);
+        if (rc != SLAPO_OK) return rc;
+    }
+    if (stages & SLAPO_BWD_DKDV) {
+#if defined(EXP_TIMING) || defined(EXP_TIMING_DQ)
+        a.dk = dk;
         a.o = g_timing_buf;
 #endif
         rc = prm->dtype == SLAPO_F16 ? attn_bwd_mfma_f16(a, st) : attn_bwd_mfma_bf16(a, st);
-        if (rc != SLAPO_OK) return rc;
     }
-    if (stages & SLAPO_BWD_DQ)
-        rc = prm->dtype == SLAPO_F16 ? attn_bwd_dq_mfma_f16(a, st) : attn_bwd_dq_mfma_bf16(a, st);
     return rc;
 }
 
