@@ -309,6 +309,9 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_fwd_kerne
     // ---- prologue: tiles 0 and 1 of this workgroup into LDS, tile 2 in flight -----------------
     // Two register stages alternate: a tile is requested two iterations before it is written to
     // LDS, so a full iteration of math sits between the request and the wait.
+    // With two workgroups per CU (DPAD <= 64) one register stage set is enough and leaves the
+    // registers to the math; a lone workgroup per CU wants the deeper prefetch of two sets.
+    constexpr bool kTwoStages = DPAD > 64;
     Stage ks_a, vs_a, ks_b, vs_b;
     // rows are clamped into the tensor, so the requests are safe whatever n_tiles is
     ks_a.load(k_base, a.ks[1], t_lo * kBN, a.sk, a.d);
@@ -329,7 +332,7 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_fwd_kerne
     for (int t = 0; t < DK; ++t)
         qf[t] = __builtin_bit_cast(
             frag_t, keep_or_zero(q_raw[t], q_row < a.sq && 16 * t + 8 * g < a.d));
-    if (2 < n_tiles) {
+    if (kTwoStages && 2 < n_tiles) {
         ks_b.load(k_base, a.ks[1], (t_lo + 2) * kBN, a.sk, a.d);
         vs_b.load(v_base, a.vs[1], (t_lo + 2) * kBN, a.sk, a.d);
     }
@@ -348,14 +351,22 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_fwd_kerne
     // finished reading it for the scores above before any wavefront gets there.
     __syncthreads();
 
-    // iteration r: requests tile r+3 into (k_ld, v_ld), writes tile r+2 from (k_st, v_st)
+    // iteration r with two stage sets: requests tile r+3 into (k_ld, v_ld), writes tile r+2 from
+    // (k_st, v_st); with one: requests tile r+2 at the top and writes it at the bottom
     auto iteration = [&](int r, f32x16_t (&s_cur)[2], f32x16_t (&s_next)[2], Stage& k_ld,
                          Stage& v_ld, Stage& k_st, Stage& v_st) __attribute__((always_inline)) {
         const int t = t_lo + r;
         TSTAMP();
-        if (r + 3 < n_tiles) {
-            k_ld.load(k_base, a.ks[1], (t + 3) * kBN, a.sk, a.d);
-            v_ld.load(v_base, a.vs[1], (t + 3) * kBN, a.sk, a.d);
+        if constexpr (kTwoStages) {
+            if (r + 3 < n_tiles) {
+                k_ld.load(k_base, a.ks[1], (t + 3) * kBN, a.sk, a.d);
+                v_ld.load(v_base, a.vs[1], (t + 3) * kBN, a.sk, a.d);
+            }
+        } else {
+            if (r + 2 < n_tiles) {
+                k_st.load(k_base, a.ks[1], (t + 2) * kBN, a.sk, a.d);
+                v_st.load(v_base, a.vs[1], (t + 2) * kBN, a.sk, a.d);
+            }
         }
         const bool next_active = tile_active(t + 1);
         const T* k_next = k_lds + ((r + 1) % kKRing) * kTileElems;
@@ -393,8 +404,13 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_fwd_kerne
     };
 
     for (int r = 0; r < n_tiles; r += 2) {
-        iteration(r, s_a, s_b, ks_a, vs_a, ks_b, vs_b);
-        if (r + 1 < n_tiles) iteration(r + 1, s_b, s_a, ks_b, vs_b, ks_a, vs_a);
+        if constexpr (kTwoStages) {
+            iteration(r, s_a, s_b, ks_a, vs_a, ks_b, vs_b);
+            if (r + 1 < n_tiles) iteration(r + 1, s_b, s_a, ks_b, vs_b, ks_a, vs_a);
+        } else {
+            iteration(r, s_a, s_b, ks_a, vs_a, ks_a, vs_a);
+            if (r + 1 < n_tiles) iteration(r + 1, s_b, s_a, ks_a, vs_a, ks_a, vs_a);
+        }
     }
 
     TSTAMP();
