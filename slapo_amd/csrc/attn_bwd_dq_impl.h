@@ -61,15 +61,6 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_dq_ke
     const int i_loc = lane & 31;
     const int wq0 = q0 + wave * 32;
     const int q_row = wq0 + i_loc;
-#ifdef EXP_TIMING_DQ
-    unsigned long long* tbuf = reinterpret_cast<unsigned long long*>(a.dk) + 512;
-    int tcount = 0;
-    const bool trec = (blockIdx.x == EXP_TIMING_DQ) && threadIdx.x == 0;
-#define TSTAMP_DQ() do { if (trec) tbuf[tcount++] = __builtin_readcyclecounter(); } while (0)
-    TSTAMP_DQ();
-#else
-#define TSTAMP_DQ() do {} while (0)
-#endif
 
     const T* q_base = reinterpret_cast<const T*>(a.q) + b * a.qs[0] + h * a.qs[2];
     const T* k_base = reinterpret_cast<const T*>(a.k) + b * a.ks[0] + h * a.ks[2];
@@ -355,7 +346,6 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_dq_ke
         constexpr bool kFast = decltype(fast_tag)::value;
         const int t = t_lo + r;
         const bool have_next = r + 1 < n_tiles;
-        TSTAMP_DQ();
         if (have_next) {
             ks.load(k_base, a.ks[1], (t + 1) * kBN, a.sk, a.d);
             vs.load(v_base, a.vs[1], (t + 1) * kBN, a.sk, a.d);
@@ -372,16 +362,13 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_dq_ke
             else
                 tile_body(kt, vt, t, std::integral_constant<int, 1>{});
         }
-        TSTAMP_DQ();
         if (have_next) {
             ks.fix((t + 1) * kBN, a.sk, a.d);
             vs.fix((t + 1) * kBN, a.sk, a.d);
             ks.store(k_lds + ((r + 1) % kKRing) * kTileElems);
             vs.store(v_lds + ((r + 1) % kVRing) * kTileElems);
         }
-        TSTAMP_DQ();
         __syncthreads();
-        TSTAMP_DQ();
     };
     // leading tiles that need neither mask nor activity test for any of the 128 queries
     int n_fast = 0;
@@ -393,8 +380,6 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_dq_ke
     int r = 0;
     for (; r < n_fast; ++r) iteration(r, std::true_type{});
     for (; r < n_tiles; ++r) iteration(r, std::false_type{});
-
-    TSTAMP_DQ();
     // ---- epilogue: dQ = scale * dQ^T^T ----
     if (q_row < a.sq) {
         T* dq_row =

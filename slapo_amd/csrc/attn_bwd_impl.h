@@ -73,15 +73,6 @@ __global__ __launch_bounds__(kBwdThreads, ((DPAD <= 64 && KB == 1) ? 2 : 1)) voi
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wavefront-uniform
     const int g = lane >> 5;
     const int c_loc = lane & 31;
-#ifdef EXP_TIMING
-    unsigned long long* tbuf = reinterpret_cast<unsigned long long*>(a.o) + 512;
-    int tcount = 0;
-    const bool trec = (blockIdx.x == EXP_TIMING) && threadIdx.x == 0;
-#define TSTAMP() do { if (trec) tbuf[tcount++] = __builtin_readcyclecounter(); } while (0)
-    TSTAMP();
-#else
-#define TSTAMP() do {} while (0)
-#endif
     const int kw0 = k0 + wave * kWaveKeys;  // first key of this wavefront
     int key[KB];                            // this lane's key column in each block
 #pragma unroll
@@ -369,7 +360,6 @@ __global__ __launch_bounds__(kBwdThreads, ((DPAD <= 64 && KB == 1) ? 2 : 1)) voi
     // body is one straight block; the others test activity and masks per wavefront and half.
     auto iteration = [&](int t, auto fast_tag) __attribute__((always_inline)) {
         constexpr bool kFast = decltype(fast_tag)::value;
-        TSTAMP();
         const int buf = (t - t_lo) & 1;
         const T* qt = q_lds + buf * SM::kQTile;
         const T* gt = g_lds + buf * SM::kQTile;
@@ -413,7 +403,6 @@ __global__ __launch_bounds__(kBwdThreads, ((DPAD <= 64 && KB == 1) ? 2 : 1)) voi
             generic_half(0);
             generic_half(1);
         }
-        TSTAMP();
         // stage the next query tile (its buffer was last read before the previous barrier)
         if (have_next) {
             qst.fix(i0 + kBwdBM, a.sq, a.d);
@@ -422,24 +411,19 @@ __global__ __launch_bounds__(kBwdThreads, ((DPAD <= 64 && KB == 1) ? 2 : 1)) voi
             gst.store(g_lds + (buf ^ 1) * SM::kQTile);
             store_stats(buf ^ 1, i0 + kBwdBM);
         }
-        TSTAMP();
         __syncthreads();
-        TSTAMP();
     };
     auto tile_fast = [&](int t) __attribute__((always_inline)) {
         const int i0 = t * kBwdBM;
         return a.window <= 0 && k0 + kBN <= a.sk && i0 + kBwdBM <= a.sq &&
                (!a.causal || i0 >= k0 + kBN - 1);
     };
-    TSTAMP();
     {
         int t = t_lo;
         for (; t < t_hi && !tile_fast(t); ++t) iteration(t, std::false_type{});
         for (; t < t_hi && tile_fast(t); ++t) iteration(t, std::true_type{});
         for (; t < t_hi; ++t) iteration(t, std::false_type{});
     }
-
-    TSTAMP();
     // ---- write dK, dV ----
 #pragma unroll
     for (int kb = 0; kb < KB; ++kb) {

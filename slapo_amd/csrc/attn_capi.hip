@@ -131,13 +131,6 @@ bool half_ptrs_ok(std::initializer_list<const void*> ptrs) {
 
 }  // namespace
 
-#if defined(EXP_TIMING) || defined(EXP_TIMING_DQ)
-void* g_timing_buf = nullptr;
-extern "C" int slapo_dbg_timing(unsigned long long* out, int n) {
-    hipDeviceSynchronize();
-    return (int)hipMemcpy(out, g_timing_buf, n * 8, hipMemcpyDeviceToHost);
-}
-#endif
 
 extern "C" int slapo_amd_attn_fwd(const slapo_attn_params* prm, const void* q, const void* k,
                                   const void* v, const float* bias, void* o, float* lse,
@@ -149,12 +142,6 @@ extern "C" int slapo_amd_attn_fwd(const slapo_attn_params* prm, const void* q, c
     a.q = q, a.k = k, a.v = v, a.o = o, a.lse = lse;
     set_bias(&a, bias);
     hipStream_t st = (hipStream_t)stream;
-#ifdef EXP_TIMING
-    {
-        if (!g_timing_buf) { hipMalloc(&g_timing_buf, 1 << 16); hipMemset(g_timing_buf, 0, 1 << 16); }
-        a.delta = (float*)g_timing_buf;
-    }
-#endif
     if (prm->dtype == SLAPO_F32) return attn_fwd_f32(a, st);
     if (!half_ptrs_ok({q, k, v, o})) return SLAPO_ERR_ALIGN;
     return prm->dtype == SLAPO_F16 ? attn_fwd_mfma_f16(a, st) : attn_fwd_mfma_bf16(a, st);
@@ -225,18 +212,10 @@ extern "C" int slapo_amd_attn_bwd_stages(const slapo_attn_params* prm, const voi
     // 16-bit types: PREPARE has nothing to do (the dQ kernel computes delta for its own rows and
     // stores it for the dK / dV kernel), so DQ runs before DKDV.
     if (stages & SLAPO_BWD_DQ) {
-#if defined(EXP_TIMING) || defined(EXP_TIMING_DQ)
-        if (!g_timing_buf) { hipMalloc(&g_timing_buf, 1 << 16); hipMemset(g_timing_buf, 0, 1 << 16); }
-        a.dk = g_timing_buf;
-#endif
         rc = prm->dtype == SLAPO_F16 ? attn_bwd_dq_mfma_f16(a, st) : attn_bwd_dq_mfma_bf16(a, st);
         if (rc != SLAPO_OK) return rc;
     }
     if (stages & SLAPO_BWD_DKDV) {
-#if defined(EXP_TIMING) || defined(EXP_TIMING_DQ)
-        a.dk = dk;
-        a.o = g_timing_buf;
-#endif
         rc = prm->dtype == SLAPO_F16 ? attn_bwd_mfma_f16(a, st) : attn_bwd_mfma_bf16(a, st);
     }
     return rc;

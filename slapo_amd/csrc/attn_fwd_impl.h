@@ -77,15 +77,6 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_fwd_kerne
     const int g = lane >> 5;
     const int i_loc = lane & 31;
     const int wq0 = q0 + wave * 32;  // first query of this wavefront
-#ifdef EXP_TIMING
-    unsigned long long* tbuf = reinterpret_cast<unsigned long long*>(a.delta);
-    int tcount = 0;
-    const bool trec = (blockIdx.x == EXP_TIMING) && threadIdx.x == 0;
-#define TSTAMP() do { if (trec) tbuf[tcount++] = __builtin_readcyclecounter(); } while (0)
-    TSTAMP();
-#else
-#define TSTAMP() do {} while (0)
-#endif
     const int q_row = wq0 + i_loc;
 
     const T* q_base = reinterpret_cast<const T*>(a.q) + b * a.qs[0] + h * a.qs[2];
@@ -337,7 +328,6 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_fwd_kerne
         vs_b.load(v_base, a.vs[1], (t_lo + 2) * kBN, a.sk, a.d);
     }
     __syncthreads();
-    TSTAMP();
 
     // Two score buffers that swap roles every iteration (no register copies).
     f32x16_t s_a[2], s_b[2];
@@ -356,7 +346,6 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_fwd_kerne
     auto iteration = [&](int r, f32x16_t (&s_cur)[2], f32x16_t (&s_next)[2], Stage& k_ld,
                          Stage& v_ld, Stage& k_st, Stage& v_st) __attribute__((always_inline)) {
         const int t = t_lo + r;
-        TSTAMP();
         if constexpr (kTwoStages) {
             if (r + 3 < n_tiles) {
                 k_ld.load(k_base, a.ks[1], (t + 3) * kBN, a.sk, a.d);
@@ -390,7 +379,6 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_fwd_kerne
         }
         if (next_active) update_reference(mx_next);
         cur_active = next_active;
-        TSTAMP();
 
         if (r + 2 < n_tiles) {
             k_st.fix((t + 2) * kBN, a.sk, a.d);
@@ -398,9 +386,7 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_fwd_kerne
             k_st.store(k_lds + ((r + 2) % kKRing) * kTileElems);
             v_st.store(v_lds + ((r + 2) % kVRing) * kTileElems);
         }
-        TSTAMP();
         __syncthreads();
-        TSTAMP();
     };
 
     for (int r = 0; r < n_tiles; r += 2) {
@@ -412,8 +398,6 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_fwd_kerne
             if (r + 1 < n_tiles) iteration(r + 1, s_b, s_a, ks_a, vs_a, ks_a, vs_a);
         }
     }
-
-    TSTAMP();
     // ---- epilogue ----
     const float l_tot = sum_xor32(l_run);
     const float inv_l = 1.0f / l_tot;

@@ -48,12 +48,8 @@ __device__ __forceinline__ Chunk<T, V> load_chunk(const T* p) {
         c.v[0] = *p;
     } else {
         static_assert(sizeof(Chunk<T, V>) == 16, "vector chunk must be 16 bytes");
-#ifdef EPI_NO_NT
-        *reinterpret_cast<u32x4_t*>(&c) = *reinterpret_cast<const u32x4_t*>(p);
-#else
         *reinterpret_cast<u32x4_t*>(&c) =
             __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(p));
-#endif
     }
     return c;
 }
@@ -72,12 +68,8 @@ __device__ __forceinline__ void store_chunk(T* p, const Chunk<T, V>& c) {
     if constexpr (V == 1) {
         *p = c.v[0];
     } else {
-#ifdef EPI_NO_NT_ST
-        *reinterpret_cast<u32x4_t*>(p) = *reinterpret_cast<const u32x4_t*>(&c);
-#else
         __builtin_nontemporal_store(*reinterpret_cast<const u32x4_t*>(&c),
                                     reinterpret_cast<u32x4_t*>(p));
-#endif
     }
 }
 
@@ -107,10 +99,7 @@ __device__ __forceinline__ uint32_t keep_bits(const DropoutState& s, uint64_t e0
 // ----------------------------------------------------------------------------------------
 // Forward kernels: flat over chunks; a block covers kUnroll * 256 consecutive chunks.
 // ----------------------------------------------------------------------------------------
-#ifndef EPI_UNROLL
-#define EPI_UNROLL 1
-#endif
-constexpr int kUnroll = EPI_UNROLL;
+constexpr int kUnroll = 1;  // chunks per thread (more did not help on MI355X)
 
 template <typename T, int V>
 __global__ __launch_bounds__(256) void bias_gelu_fwd_kernel(const T* __restrict__ y,
@@ -143,15 +132,13 @@ __global__ __launch_bounds__(256) void bias_gelu_fwd_kernel(const T* __restrict_
     }
 }
 
-#ifndef EPI_DROP_UNROLL
-#define EPI_DROP_UNROLL 1
-#endif
+constexpr int kDropUnroll = 1;  // chunks per thread of the dropout forward kernel
 template <typename T, int V, bool kResidual, int kDrop>
 __global__ __launch_bounds__(256) void bias_dropout_residual_fwd_kernel(
     const T* __restrict__ x, const T* __restrict__ bias, const T* __restrict__ residual,
     T* __restrict__ out, uint64_t n_chunks, uint32_t chunks_per_row, uint32_t row_mask,
     DropoutState s) {
-    constexpr int kDU = EPI_DROP_UNROLL;
+    constexpr int kDU = kDropUnroll;
     const uint64_t base = (uint64_t)blockIdx.x * (256 * kDU) + threadIdx.x;
     Chunk<T, V> in[kDU];
     Chunk<T, V> res[kDU];
@@ -189,10 +176,7 @@ __global__ __launch_bounds__(256) void bias_dropout_residual_fwd_kernel(
 // keeping per-thread fp32 column sums; the 4 row-lanes are combined through LDS and written
 // as one fp32 partial row per block.
 // ----------------------------------------------------------------------------------------
-#ifndef EPI_ROWS
-#define EPI_ROWS 64
-#endif
-constexpr int kRowsPerBlock = EPI_ROWS;
+constexpr int kRowsPerBlock = 64;
 constexpr int kRowLanes = 4;
 constexpr int kColLanes = 64;
 
@@ -373,7 +357,7 @@ int dropres_fwd_launch(const void* x, const void* bias, const void* residual, vo
                        int64_t rows, int64_t cols, bool dropout, const DropoutState& s,
                        hipStream_t st) {
     RowGeom g;
-    if (!flat_geom(rows, cols, V, &g, EPI_DROP_UNROLL)) return SLAPO_ERR_SHAPE;
+    if (!flat_geom(rows, cols, V, &g, kDropUnroll)) return SLAPO_ERR_SHAPE;
 #define SLAPO_LAUNCH_DR(RES, DROP)                                                             \
     hipLaunchKernelGGL((bias_dropout_residual_fwd_kernel<T, V, RES, DROP>), dim3(g.blocks),    \
                        dim3(256), 0, st, (const T*)x, (const T*)bias, (const T*)residual,      \
