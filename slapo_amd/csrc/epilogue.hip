@@ -272,33 +272,40 @@ __global__ __launch_bounds__(256) void bias_dropout_bwd_kernel(const T* __restri
                       });
 }
 
-// Second stage of the column reduction: a block owns 64 columns; its 4 row-lanes walk the partial
-// rows with a stride of 4 (coalesced 256-byte reads), then combine through LDS.
+// Second stage of the column reduction: a block owns 16 columns; its 16 row-lanes walk the partial
+// rows with a stride of 16 (64-byte segments; the whole partial matrix is a few MB), then combine
+// through LDS.  Many small blocks: the stage is latency bound, not bandwidth bound.
+constexpr int kFinCols = 16;
+constexpr int kFinRows = 16;
 template <typename T>
 __global__ __launch_bounds__(256) void colsum_finish_kernel(const float* __restrict__ partial,
                                                             T* __restrict__ dbias,
                                                             int64_t n_partials, int64_t cols) {
-    __shared__ float red[kRowLanes][kColLanes];
-    const int cx = threadIdx.x % kColLanes;
-    const int ry = threadIdx.x / kColLanes;
-    const int64_t c = (int64_t)blockIdx.x * kColLanes + cx;
+    __shared__ float red[kFinRows][kFinCols + 1];
+    const int cx = threadIdx.x % kFinCols;
+    const int ry = threadIdx.x / kFinCols;
+    const int64_t c = (int64_t)blockIdx.x * kFinCols + cx;
     float t = 0.f;
     if (c < cols) {
         float t0 = 0.f, t1 = 0.f, t2 = 0.f, t3 = 0.f;
         int64_t k = ry;
-        for (; k + 3 * kRowLanes < n_partials; k += 4 * kRowLanes) {
+        for (; k + 3 * kFinRows < n_partials; k += 4 * kFinRows) {
             t0 += partial[k * cols + c];
-            t1 += partial[(k + kRowLanes) * cols + c];
-            t2 += partial[(k + 2 * kRowLanes) * cols + c];
-            t3 += partial[(k + 3 * kRowLanes) * cols + c];
+            t1 += partial[(k + kFinRows) * cols + c];
+            t2 += partial[(k + 2 * kFinRows) * cols + c];
+            t3 += partial[(k + 3 * kFinRows) * cols + c];
         }
-        for (; k < n_partials; k += kRowLanes) t0 += partial[k * cols + c];
+        for (; k < n_partials; k += kFinRows) t0 += partial[k * cols + c];
         t = (t0 + t1) + (t2 + t3);
     }
     red[ry][cx] = t;
     __syncthreads();
-    if (ry == 0 && c < cols)
-        dbias[c] = Elem<T>::from_f32((red[0][cx] + red[1][cx]) + (red[2][cx] + red[3][cx]));
+    if (ry == 0 && c < cols) {
+        float sum = 0.f;
+#pragma unroll
+        for (int r = 0; r < kFinRows; ++r) sum += red[r][cx];
+        dbias[c] = Elem<T>::from_f32(sum);
+    }
 }
 
 // ----------------------------------------------------------------------------------------
@@ -393,7 +400,7 @@ inline bool bwd_grid(int64_t rows, int64_t cols, int v, dim3* grid) {
 template <typename T>
 int finish_colsum(const float* partial, void* dbias, int64_t rows, int64_t cols, hipStream_t st) {
     const int64_t n_partials = (rows + kRowsPerBlock - 1) / kRowsPerBlock;
-    const unsigned blocks = (unsigned)((cols + kColLanes - 1) / kColLanes);
+    const unsigned blocks = (unsigned)((cols + kFinCols - 1) / kFinCols);
     hipLaunchKernelGGL((colsum_finish_kernel<T>), dim3(blocks), dim3(256), 0, st, partial,
                        (T*)dbias, n_partials, cols);
     return check_launch();

@@ -208,3 +208,42 @@ def test_full_size_cfg2_properties():
     a_ = (qh.grad.double() * q.double()).sum(dim=(1, 3))
     b_ = (kh.grad.double() * k.double()).sum(dim=(1, 3))
     assert ((a_ - b_).abs().max() / a_.abs().max()).item() <= 2e-2
+
+
+def test_backward_is_bitwise_reproducible_and_stages_compose():
+    """The backward keeps no accumulator in memory and uses no atomics: two runs give identical
+    bits; running the stages one by one (PREPARE, DQ, DKDV) equals the single call."""
+    import ctypes
+
+    from slapo_amd import _lib
+    from slapo_amd.op import _kernels as K
+
+    lib = _lib.load()
+    q, k, v, do, _ = _inputs(2, 320, 4, 64, torch.bfloat16)
+    q, k, v, do = (t.cuda() for t in (q, k, v, do))
+    o, lse, _ = K.attn_fwd(q, k, v, None, True, 0, 64 ** -0.5, 0.0, 1, 0, None)
+    prm = K.make_attn_params(q, k, v, o, None, True, 0, 64 ** -0.5, 0.0, 1, 0, None)
+    nb = lib.slapo_amd_attn_bwd_workspace_bytes(ctypes.byref(prm))
+    assert nb == 2 * 4 * 320 * 4  # delta only: one fp32 per (batch, head, query)
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+
+    def run(stage_list):
+        ws = torch.full((nb // 4,), float("nan"), device="cuda")
+        dq, dk, dv = (torch.full_like(q, float("nan")) for _ in range(3))
+        strides = [K._bshd_strides(t) for t in (dq, dk, dv)]
+        for stages in stage_list:
+            rc = lib.slapo_amd_attn_bwd_stages(ctypes.byref(prm), P(q), P(k), P(v), None, P(o),
+                                               P(do), P(lse), P(dq), P(dk), P(dv), *strides,
+                                               P(ws), nb, stages, st)
+            assert rc == 0
+        torch.cuda.synchronize()
+        return dq, dk, dv
+
+    first = run([_lib.BWD_ALL])
+    again = run([_lib.BWD_ALL])
+    staged = run([_lib.BWD_PREPARE, _lib.BWD_DQ, _lib.BWD_DKDV])
+    for a, b_, c in zip(first, again, staged):
+        assert not torch.isnan(a.float()).any()
+        assert torch.equal(a, b_)
+        assert torch.equal(a, c)
