@@ -114,6 +114,24 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_dq_ke
         delta = sum_xor32(part);  // masked dO slots are zero, so clamped rows / columns add nothing
         if (row_ok && g == 0) a.delta[(int64_t)bh * a.sq + q_row] = delta;
     }
+    // Without dropout dP^T - delta comes straight out of the matrix pipe: one extra k-step whose A
+    // operand is 1 in k-slots 0..2 (every key row alike) and whose B operand holds -delta of this
+    // lane's query, split into three parts of T whose sum carries at least 24 bits of it, i.e. the
+    // subtraction is as exact as in fp32.
+    frag_t ones_f, ndelta_f;
+    {
+        const float nd = -delta;
+        const T hi = (T)nd;
+        const float r1 = nd - (float)hi;
+        const T mid = (T)r1;
+        const T lo = (T)(r1 - (float)mid);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) ones_f[j] = (T)0.f, ndelta_f[j] = (T)0.f;
+        if (g == 0) {
+            ones_f[0] = (T)1.f, ones_f[1] = (T)1.f, ones_f[2] = (T)1.f;
+            ndelta_f[0] = hi, ndelta_f[1] = mid, ndelta_f[2] = lo;
+        }
+    }
 
     f32x16_t dq_acc[DV];
 #pragma unroll
@@ -166,6 +184,7 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_dq_ke
 #pragma unroll
         for (int x = 0; x < DK; ++x)
             dp = Mma<T>::mma32(lds_frag<T>(vt + kb * 32 * kPitch + row_off + 16 * x), gf[x], dp);
+        if constexpr (kDrop == 0) dp = Mma<T>::mma32(ones_f, ndelta_f, dp);
     };
     // dQ^T += K_half^T dS^T half
     auto half_dq = [&](const T* kt, int kb, const uint32_t (&dw)[8]) __attribute__((always_inline)) {
@@ -246,7 +265,10 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_dq_ke
             for (int e = 0; e < 4; ++e) {
                 float d = dp[4 * r4 + e];
                 if constexpr (kDrop != 0) d = ((bits >> e) & 1u) ? d * a.rng.inv_keep : 0.f;
-                dv[e] = p[4 * r4 + e] * (d - delta);
+                if constexpr (kDrop == 0)
+                    dv[e] = p[4 * r4 + e] * d;  // delta already subtracted by the matrix pipe
+                else
+                    dv[e] = p[4 * r4 + e] * (d - delta);
             }
             dw[2 * r4] = pack2<T>(dv[0], dv[1]);
             dw[2 * r4 + 1] = pack2<T>(dv[2], dv[3]);
@@ -314,6 +336,7 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_dq_ke
         __builtin_amdgcn_sched_barrier(0);
         rows(vt, 1, vr1);
         mma_rows(vr0, gf, p0);
+        if constexpr (kDrop == 0) p0 = Mma<T>::mma32(ones_f, ndelta_f, p0);
         __builtin_amdgcn_sched_barrier(0);
         cols(0, kq0);
         mma_rows(kr1, qf, s1);
@@ -321,6 +344,7 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_dq_ke
         __builtin_amdgcn_sched_barrier(0);
         cols(1, kq1);
         mma_rows(vr1, gf, p1);
+        if constexpr (kDrop == 0) p1 = Mma<T>::mma32(ones_f, ndelta_f, p1);
         half_ds(s0, p0, t, 0, dw0);
         __builtin_amdgcn_sched_barrier(0);
         mma_cols(kq0, dw0);
