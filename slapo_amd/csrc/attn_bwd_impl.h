@@ -127,6 +127,31 @@ __global__ __launch_bounds__(kBwdThreads, ((DPAD <= 64 && KB == 1) ? 2 : 1)) voi
         }
     }
     const float c_log2 = a.scale_log2;
+    // Folding the per-row terms into the matrix pipe (below) pays where a workgroup has the CU to
+    // itself (DPAD > 64: 3 % faster); at DPAD 64 its extra registers spill and it measured slower.
+    constexpr bool kFold = DPAD > 64;
+    const float inv_scale = 1.0f / a.scale;
+    constexpr float kNoRow = 30000.f;  // fits fp16; scale_log2 * (s - kNoRow) underflows exp2
+
+    // The per-row terms (- lse / scale for S, - delta for dP) are added by the matrix pipe: one
+    // extra k-step whose A operand holds the term of each query row, split into three parts of T
+    // (their sum carries 24 bits) in k-slots 0..2, and whose B operand is 1 in those slots.
+    frag_t ones_f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) ones_f[j] = (T)0.f;
+    if (g == 0) ones_f[0] = (T)1.f, ones_f[1] = (T)1.f, ones_f[2] = (T)1.f;
+    auto row_term = [&](float v) __attribute__((always_inline)) {
+        const float nv = -v;
+        const T hi = (T)nv;
+        const float r1 = nv - (float)hi;
+        const T mid = (T)r1;
+        const T lo = (T)(r1 - (float)mid);
+        frag_t f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) f[j] = (T)0.f;
+        if (g == 0) f[0] = hi, f[1] = mid, f[2] = lo;
+        return f;
+    };
 
     // per-lane LDS offsets (elements) that do not change from tile to tile
     const int a_off = pi_row(c_loc) * kPitch + 8 * g;
@@ -144,9 +169,19 @@ __global__ __launch_bounds__(kBwdThreads, ((DPAD <= 64 && KB == 1) ? 2 : 1)) voi
     auto store_stats = [&](int buf, int i0) __attribute__((always_inline)) {
         if (threadIdx.x < 2 * kBwdBM) {
             const bool ok = i0 + (int)(threadIdx.x & (kBwdBM - 1)) < a.sq;
-            // lse in log2 units, +inf for rows past the end so that P = 0 there; delta 0
-            float v = (threadIdx.x < kBwdBM) ? (ok ? stat_reg * kLog2e : INFINITY)
-                                             : (ok ? stat_reg : 0.f);
+            // lse in units of the raw dot product (lse / scale), so that exp2(scale_log2 * (s - lse))
+            // is the probability; a large finite value for rows past the end so that P = 0 there;
+            // delta 0
+            // (clamped: a row without any visible key has lse = -inf, and the three-way split
+            // needs finite input)
+            float v;
+            if constexpr (kFold)
+                v = (threadIdx.x < kBwdBM)
+                        ? (ok ? fmaxf(fminf(stat_reg * inv_scale, kNoRow), -kNoRow) : kNoRow)
+                        : (ok ? stat_reg : 0.f);
+            else  // lse in log2 units, +inf past the end
+                v = (threadIdx.x < kBwdBM) ? (ok ? stat_reg * kLog2e : INFINITY)
+                                           : (ok ? stat_reg : 0.f);
             stat_lds[buf * 2 * kBwdBM + threadIdx.x] = v;
         }
     };
@@ -188,8 +223,8 @@ __global__ __launch_bounds__(kBwdThreads, ((DPAD <= 64 && KB == 1) ? 2 : 1)) voi
 
     // ---- stages of one half tile (32 queries at ih0 = i0 + 32 hf) ----
     // S = Q_h K_w^T, dP = dO_h V_w^T: every Q / dO fragment read feeds KB matrix instructions
-    auto half_sp = [&](const T* qt, const T* gt, int hf, f32x16_t (&s)[KB], f32x16_t (&dp)[KB])
-                       __attribute__((always_inline)) {
+    auto half_sp = [&](const T* qt, const T* gt, const float* lse_h, const float* delta_h, int hf,
+                       f32x16_t (&s)[KB], f32x16_t (&dp)[KB]) __attribute__((always_inline)) {
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
@@ -204,6 +239,17 @@ __global__ __launch_bounds__(kBwdThreads, ((DPAD <= 64 && KB == 1) ? 2 : 1)) voi
             for (int kb = 0; kb < KB; ++kb) {
                 s[kb] = Mma<T>::mma32(qa, kf[kb][x], s[kb]);
                 dp[kb] = Mma<T>::mma32(ga, vf[kb][x], dp[kb]);
+            }
+        }
+        if constexpr (kFold) {
+            // A-operand row of this lane is query pi(c_loc) of the half
+            const frag_t lse_a = row_term(lse_h[pi_row(c_loc)]);
+#pragma unroll
+            for (int kb = 0; kb < KB; ++kb) s[kb] = Mma<T>::mma32(lse_a, ones_f, s[kb]);
+            if constexpr (kDrop == 0) {
+                const frag_t del_a = row_term(delta_h[pi_row(c_loc)]);
+#pragma unroll
+                for (int kb = 0; kb < KB; ++kb) dp[kb] = Mma<T>::mma32(del_a, ones_f, dp[kb]);
             }
         }
     };
@@ -225,12 +271,17 @@ __global__ __launch_bounds__(kBwdThreads, ((DPAD <= 64 && KB == 1) ? 2 : 1)) voi
 #pragma unroll
         for (int r4 = 0; r4 < 4; ++r4) {
             const int qoff = acc_row(4 * r4, g);
-            const f32x4_t lse4 = *reinterpret_cast<const f32x4_t*>(lse_h + qoff);
+            f32x4_t lse4 = {0.f, 0.f, 0.f, 0.f};
+            if constexpr (!kFold) lse4 = *reinterpret_cast<const f32x4_t*>(lse_h + qoff);
 #pragma unroll
             for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    float x = __builtin_fmaf(s[kb][4 * r4 + e], c_log2, -lse4[e]);
+                    float x;
+                    if constexpr (kFold)
+                        x = s[kb][4 * r4 + e] * c_log2;  // lse already subtracted
+                    else
+                        x = __builtin_fmaf(s[kb][4 * r4 + e], c_log2, -lse4[e]);
                     if constexpr (kBias) {
                         const int i = ih0 + qoff + e;
                         if (bias_per_key)
@@ -302,7 +353,9 @@ __global__ __launch_bounds__(kBwdThreads, ((DPAD <= 64 && KB == 1) ? 2 : 1)) voi
 #pragma unroll
         for (int r4 = 0; r4 < 4; ++r4) {
             const int qoff = acc_row(4 * r4, g);
-            const f32x4_t del4 = *reinterpret_cast<const f32x4_t*>(delta_h + qoff);
+            f32x4_t del4 = {0.f, 0.f, 0.f, 0.f};  // folded and no dropout: already subtracted
+            if constexpr (kDrop != 0 || !kFold)
+                del4 = *reinterpret_cast<const f32x4_t*>(delta_h + qoff);
 #pragma unroll
             for (int kb = 0; kb < KB; ++kb) {
                 float pv[4], dv[4];
@@ -376,9 +429,9 @@ __global__ __launch_bounds__(kBwdThreads, ((DPAD <= 64 && KB == 1) ? 2 : 1)) voi
             std::integral_constant<int, 0> none;
             f32x16_t s0[KB], s1[KB], p0[KB], p1[KB];
             uint32_t pw0[KB][8], dw0[KB][8], pw1[KB][8], dw1[KB][8];
-            half_sp(qt, gt, 0, s0, p0);
+            half_sp(qt, gt, lse_t, delta_t, 0, s0, p0);
             half_exp(s0, lse_t, i0, none);
-            half_sp(qt, gt, 1, s1, p1);
+            half_sp(qt, gt, lse_t + 32, delta_t + 32, 1, s1, p1);
             half_ds(s0, p0, delta_t, i0, pw0, dw0);
             half_exp(s1, lse_t + 32, i0 + 32, none);
             half_out(qt, gt, 0, pw0, dw0);
@@ -390,7 +443,7 @@ __global__ __launch_bounds__(kBwdThreads, ((DPAD <= 64 && KB == 1) ? 2 : 1)) voi
                 if (!half_active(ih0)) return;
                 f32x16_t s[KB], dp[KB];
                 uint32_t pw[KB][8], dw[KB][8];
-                half_sp(qt, gt, hf, s, dp);
+                half_sp(qt, gt, lse_t + 32 * hf, delta_t + 32 * hf, hf, s, dp);
                 if (!half_needs_mask(ih0))
                     half_exp(s, lse_t + 32 * hf, ih0, std::integral_constant<int, 0>{});
                 else if (a.window > 0)
