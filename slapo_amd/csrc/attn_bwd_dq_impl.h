@@ -73,6 +73,9 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_dq_ke
     Stage ks, vs;
     int j_lo, j_hi;
     key_range(a, q0, min(q0 + kBM, a.sq), j_lo, j_hi);
+    if constexpr (kBias)  // skip the tiles that hold nothing but padded keys
+        j_hi = max(j_lo + 1, min(j_hi, padded_key_limit<kThreads>(
+                                           a, b, h, reinterpret_cast<float*>(smem_raw))));
     const int t_lo = j_lo / kBN;
     const int t_hi = (j_hi + kBN - 1) / kBN;
     const int n_tiles = t_hi - t_lo;

@@ -111,6 +111,10 @@ __global__ __launch_bounds__(kBwdThreads, ((DPAD <= 64 && KB == 1) ? 2 : 1)) voi
 
     int i_lo, i_hi;
     query_range(a, k0, min(k0 + kBN, a.sk), i_lo, i_hi);
+    if constexpr (kBias) {  // a workgroup that owns nothing but padded keys has dK = dV = 0
+        if (k0 >= padded_key_limit<kBwdThreads>(a, b, h, reinterpret_cast<float*>(smem_raw)))
+            i_hi = i_lo;
+    }
     const int t_lo = i_lo / kBwdBM;
     const int t_hi = (i_hi + kBwdBM - 1) / kBwdBM;
 

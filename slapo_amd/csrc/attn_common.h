@@ -165,6 +165,34 @@ __device__ __forceinline__ void query_range(const AttnArgs& a, int k_lo, int k_h
     i_hi = a.window > 0 ? min(a.sq, k_hi - 1 + a.window) : a.sq;
 }
 
+// Key-padding masks arrive as an additive bias that does not depend on the query
+// ([B,1,1,Sk] with a large negative value on padded keys).  Keys past the last unmasked one
+// contribute exp(-huge) = 0 exactly to every row that sees at least one unmasked key, so whole
+// tiles of them can be skipped.  Returns one past the last key worth visiting (a.sk when the
+// shortcut does not apply): only per-key biases, no local window, and key 0 unmasked, which
+// guarantees an unmasked visible key for every query row under a causal or full mask.
+// Called by all threads of the workgroup; `scratch` is 4 floats of LDS that nothing else uses
+// until the call returns.
+constexpr float kMaskedBias = -30000.f;  // below fp16's most negative value, far beyond any score
+template <int THREADS>
+__device__ __forceinline__ int padded_key_limit(const AttnArgs& a, int b, int h, float* scratch) {
+    if (!a.has_bias || a.bs[2] != 0 || a.window > 0) return a.sk;
+    const float* brow = a.bias + b * a.bs[0] + h * a.bs[1];
+    if (!(brow[0] > kMaskedBias)) return a.sk;
+    int last = 0;
+    for (int j = threadIdx.x; j < a.sk; j += THREADS)
+        if (brow[(int64_t)j * a.bs[3]] > kMaskedBias) last = j;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) last = max(last, __shfl_xor(last, off, 64));
+    if ((threadIdx.x & 63) == 0) scratch[threadIdx.x >> 6] = __int_as_float(last);
+    __syncthreads();
+    int limit = 0;
+#pragma unroll
+    for (int w = 0; w < THREADS / 64; ++w) limit = max(limit, __float_as_int(scratch[w]));
+    __syncthreads();
+    return limit + 1;
+}
+
 // Stage a [ROWS x DPAD] tile of T (rows row0.., zero beyond n_rows / beyond d) through registers.
 // The global loads are unconditional (out-of-range rows are clamped to the last valid row and
 // zeroed when the tile is written to LDS), so they stay in the caller's basic block and the
