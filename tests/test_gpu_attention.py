@@ -107,6 +107,31 @@ def test_additive_masks(dtype, layout):
     _check(q, k, v, do, mask, True, 0, dtype)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("kind", ["short", "left", "holes"])
+def test_padding_masks_and_tile_skipping(dtype, causal, kind):
+    """Key-padding as a per-key additive mask: valid lengths far below Sk (whole key tiles hold
+    only padding and are skipped), left padding (key 0 masked: nothing may be skipped) and
+    masked holes in the middle."""
+    b, s, h, d = 3, 320, 2, 64
+    q, k, v, do, g = _inputs(b, s, h, d, dtype)
+    neg = torch.finfo(dtype).min
+    m = torch.zeros(b, 1, 1, s)
+    if kind == "short":
+        for i, n in enumerate((70, 129, 320)):
+            m[i, 0, 0, n:] = neg
+    elif kind == "left":
+        if causal:
+            pytest.skip("rows that see only masked keys have no defined value in the reference")
+        for i, n in enumerate((5, 64, 200)):
+            m[i, 0, 0, :n] = neg
+    else:
+        m[:, 0, 0, 100:260] = neg
+        m[1, 0, 0, 300:] = neg
+    _check(q, k, v, do, m.to(dtype), causal, 0, dtype)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("window", [1, 7, 64, 100, 4096])
 def test_local_window(dtype, window):
