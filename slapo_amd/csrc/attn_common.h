@@ -130,7 +130,7 @@ struct AttnArgs {
     const void* v;
     void* o;
     const void* dout;
-    void* dq;  // fp32 accumulator in the MFMA backward, element type T in the fp32 kernels
+    void* dq;  // element type of the tensors
     void* dk;
     void* dv;
     const float* bias;
