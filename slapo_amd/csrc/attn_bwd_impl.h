@@ -424,11 +424,18 @@ __global__ __launch_bounds__(kBwdThreads, ((DPAD <= 64 && KB == 1) ? 2 : 1)) voi
         const float* delta_t = lse_t + kBwdBM;
         const int i0 = t * kBwdBM;
         const bool have_next = t + 1 < t_hi;
-        if (have_next) {
+        // The next tile is requested unconditionally (rows are clamped into the tensor; after the
+        // last tile the request is wasted) so that the request stays straight-line code.  In the
+        // fast body it is issued in the middle, once the score registers of the first half are
+        // dead, which keeps the staging registers out of the busiest stretch.
+        auto request_next = [&]() __attribute__((always_inline)) {
             qst.load(q_base, a.qs[1], i0 + kBwdBM, a.sq, a.d);
             gst.load(g_base, a.os[1], i0 + kBwdBM, a.sq, a.d);
             load_stats(i0 + kBwdBM);
-        }
+        };
+        // (only where two workgroups share a CU and registers are the scarce resource)
+        constexpr bool kLateRequest = kFast && DPAD <= 64;
+        if constexpr (!kLateRequest) request_next();
         if constexpr (kFast) {
             std::integral_constant<int, 0> none;
             f32x16_t s0[KB], s1[KB], p0[KB], p1[KB];
@@ -438,6 +445,11 @@ __global__ __launch_bounds__(kBwdThreads, ((DPAD <= 64 && KB == 1) ? 2 : 1)) voi
             half_sp(qt, gt, lse_t + 32, delta_t + 32, 1, s1, p1);
             half_ds(s0, p0, delta_t, i0, pw0, dw0);
             half_exp(s1, lse_t + 32, i0 + 32, none);
+            if constexpr (kLateRequest) {
+                __builtin_amdgcn_sched_barrier(0);
+                request_next();
+                __builtin_amdgcn_sched_barrier(0);
+            }
             half_out(qt, gt, 0, pw0, dw0);
             half_ds(s1, p1, delta_t + 32, i0 + 32, pw1, dw1);
             half_out(qt, gt, 1, pw1, dw1);
