@@ -461,7 +461,6 @@ int dispatch_flags(const AttnArgs& a, hipStream_t st) {
 
 template <typename T>
 int dispatch(const AttnArgs& a, hipStream_t st) {
-    if (a.d <= 64) return dispatch_flags<T, 64>(a, st);
     if (a.d <= 96) return dispatch_flags<T, 96>(a, st);
     if (a.d <= 128) return dispatch_flags<T, 128>(a, st);
     return SLAPO_ERR_SHAPE;
