@@ -32,8 +32,10 @@ constexpr int kBN = 64;
 constexpr int kKRing = 2;
 constexpr int kVRing = 2;
 
-template <typename T, int DPAD, bool kBias, int kDrop>
-__global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_dq_kernel(
+// kStagger: see the tile bodies below.  Staggered halves need one workgroup per CU above
+// head_dim 64; sequential halves fit two.
+template <typename T, int DPAD, bool kBias, int kDrop, bool kStagger>
+__global__ __launch_bounds__(kThreads, (kStagger && DPAD > 64 ? 1 : 2)) void attn_bwd_dq_kernel(
     const AttnArgs a) {
     typedef typename Mma<T>::frag frag_t;
     typedef TileStage<T, DPAD, kBN, kThreads> Stage;
@@ -168,9 +170,13 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_dq_ke
                (a.window > 0 && wq_last - j0 >= a.window);
     };
 
-    // The tile is processed as two halves of 32 keys whose stages are staggered, so that the matrix
-    // instructions of one half always have independent vector work of the other half around them
-    // (a wavefront overlaps the two only when they are interleaved in its instruction stream).
+    // The tile is processed as two halves of 32 keys.  With kStagger their stages are staggered,
+    // so that the matrix instructions of one half always have independent vector work of the
+    // other half around them (a wavefront overlaps the two only when they are interleaved in its
+    // instruction stream).  Without it the halves run one after the other: above head_dim 64 that
+    // is what fits two workgroups per CU into the register file, and the second resident workgroup
+    // hides more latency than the stagger does (measured: 28 % faster at head_dim 80, 2-12 % at
+    // 128; only the masked tile bodies of a local window lose, to register spills, at 128).
 
     // S^T half = K_half Q^T
     auto half_s = [&](const T* kt, int kb, f32x16_t& s) __attribute__((always_inline)) {
@@ -278,6 +284,19 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_dq_ke
         }
     };
     auto tile_body = [&](const T* kt, const T* vt, int t, auto mask_tag) __attribute__((always_inline)) {
+        if constexpr (!kStagger) {
+            f32x16_t s0, p0;
+            uint32_t dw0[8];
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+                half_s(kt, kb, s0);
+                half_dp(vt, kb, p0);
+                half_exp(s0, t, kb, mask_tag);
+                half_ds(s0, p0, t, kb, dw0);
+                half_dq(kt, kb, dw0);
+            }
+            return;
+        }
         f32x16_t s0, s1, p0, p1;
         uint32_t dw0[8], dw1[8];
         half_s(kt, 0, s0);
@@ -380,7 +399,10 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_dq_ke
         const T* kt = k_lds + (r % kKRing) * kTileElems;
         const T* vt = v_lds + (r % kVRing) * kTileElems;
         if constexpr (kFast) {
-            tile_body_fast(kt, vt, t);
+            if constexpr (kStagger)
+                tile_body_fast(kt, vt, t);
+            else
+                tile_body(kt, vt, t, std::integral_constant<int, 0>{});
         } else if (tile_active(t)) {
             if (!tile_needs_mask(t))
                 tile_body(kt, vt, t, std::integral_constant<int, 0>{});
@@ -426,14 +448,14 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 ? 2 : 1)) void attn_bwd_dq_ke
     }
 }
 
-template <typename T, int DPAD, bool kBias, int kDrop>
+template <typename T, int DPAD, bool kBias, int kDrop, bool kStagger>
 int launch(const AttnArgs& a, hipStream_t st) {
     typedef TileStage<T, DPAD, kBN, kThreads> Stage;
     const size_t smem = (size_t)(kKRing + kVRing) * kBN * Stage::kPitch * sizeof(T);
     const int n_qt = (a.sq + kBM - 1) / kBM;
     const int64_t blocks = (int64_t)n_qt * a.batch * a.heads;
     if (blocks <= 0 || blocks > 0x7FFFFFFF) return SLAPO_ERR_SHAPE;
-    auto kern = attn_bwd_dq_kernel<T, DPAD, kBias, kDrop>;
+    auto kern = attn_bwd_dq_kernel<T, DPAD, kBias, kDrop, kStagger>;
     if (smem > 48 * 1024) {
         static bool raised = false;  // per instantiation
         if (!raised) {
@@ -448,23 +470,27 @@ int launch(const AttnArgs& a, hipStream_t st) {
     return check_launch();
 }
 
-template <typename T, int DPAD>
+template <typename T, int DPAD, bool kStagger>
 int dispatch_flags(const AttnArgs& a, hipStream_t st) {
     if (a.has_bias) {
-        if (a.dropout == 1) return launch<T, DPAD, true, 1>(a, st);
-        if (a.dropout == 2) return launch<T, DPAD, true, 2>(a, st);
-        return launch<T, DPAD, true, 0>(a, st);
+        if (a.dropout == 1) return launch<T, DPAD, true, 1, kStagger>(a, st);
+        if (a.dropout == 2) return launch<T, DPAD, true, 2, kStagger>(a, st);
+        return launch<T, DPAD, true, 0, kStagger>(a, st);
     }
-    if (a.dropout == 1) return launch<T, DPAD, false, 1>(a, st);
-    if (a.dropout == 2) return launch<T, DPAD, false, 2>(a, st);
-    return launch<T, DPAD, false, 0>(a, st);
+    if (a.dropout == 1) return launch<T, DPAD, false, 1, kStagger>(a, st);
+    if (a.dropout == 2) return launch<T, DPAD, false, 2, kStagger>(a, st);
+    return launch<T, DPAD, false, 0, kStagger>(a, st);
 }
 
 template <typename T>
 int dispatch(const AttnArgs& a, hipStream_t st) {
-    if (a.d <= 64) return dispatch_flags<T, 64>(a, st);
-    if (a.d <= 96) return dispatch_flags<T, 96>(a, st);
-    if (a.d <= 128) return dispatch_flags<T, 128>(a, st);
+    if (a.d <= 64) return dispatch_flags<T, 64, true>(a, st);
+    if (a.d <= 96) return dispatch_flags<T, 96, false>(a, st);
+    if (a.d <= 128) {
+        // a local window leaves mostly masked tiles, whose bodies spill at two workgroups per CU
+        if (a.window > 0) return dispatch_flags<T, 128, true>(a, st);
+        return dispatch_flags<T, 128, false>(a, st);
+    }
     return SLAPO_ERR_SHAPE;
 }
 
