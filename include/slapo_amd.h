@@ -147,7 +147,9 @@ typedef struct slapo_attn_params {
     float p_drop;     /* dropout probability on the attention matrix; 0 disables                */
     uint64_t seed;    /* Philox seed (generator seed)                                           */
     uint64_t offset;  /* Philox offset (generator offset at entry of forward)                   */
-    /* element strides of [batch, seqlen, heads] for each tensor; head_dim stride is 1 */
+    /* element strides of [batch, seqlen, heads] for each tensor; head_dim stride is 1.  For the
+     * 16-bit types: multiples of 8, and the seqlen stride in [0, 2^24) (SLAPO_ERR_ALIGN /
+     * SLAPO_ERR_SHAPE otherwise) */
     int64_t q_strides[3];
     int64_t k_strides[3];
     int64_t v_strides[3];

@@ -162,6 +162,8 @@ __global__ __launch_bounds__(kBwdThreads, ((DPAD <= 64 && KB == 1) ? 2 : 1)) voi
     const int t_off = (8 * g + ((lane & 15) >> 2)) * kPitch + ((lane >> 4) & 1) * 16 + 4 * (lane & 3);
 
     QStage qst, gst;
+    qst.init(a.qs[1], a.d);
+    gst.init(a.os[1], a.d);
     // lse / delta of a query tile: threads 0..63 fetch lse, threads 64..127 delta.  The load is
     // unconditional (row clamped) and its result is not touched until the tile is written to LDS.
     float stat_reg = 0.f;

@@ -84,6 +84,9 @@ int fill_args(const slapo_attn_params* p, AttnArgs* a, bool backward) {
         if (!strides_ok(p->q_strides, 8) || !strides_ok(p->k_strides, 8) ||
             !strides_ok(p->v_strides, 8) || !strides_ok(p->o_strides, 8))
             return SLAPO_ERR_ALIGN;
+        // the tile loads address rows with 32-bit byte offsets from a per-tile base
+        for (const int64_t* st : {p->q_strides, p->k_strides, p->v_strides, p->o_strides})
+            if (st[1] < 0 || st[1] >= (int64_t(1) << 24)) return SLAPO_ERR_SHAPE;
     }
     for (int i = 0; i < 3; ++i) {
         a->qs[i] = p->q_strides[i];

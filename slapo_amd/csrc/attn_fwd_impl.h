@@ -1,0 +1,396 @@
+// Flash-attention forward for gfx950 (fp16 / bf16 inputs, fp32 accumulation).
+//
+// One workgroup (4 wavefronts) owns 128 consecutive queries of one (batch, head); wavefront w owns
+// 32 of them, lane l = one query (lanes l and l + 32 share a query and split the registers' keys
+// resp. head-dim slots).  Keys and values stream through LDS in tiles of 64, double buffered and
+// staged through registers (the global loads of tile t+1 are in flight while tile t is
+// processed).  Per key tile, as two halves of 32 keys:
+//   S^T  = K Q^T                  A = K rows from LDS (row-permuted 128-bit reads), B = Q^T regs
+//   P^T  = exp2(S^T * scale - m)  online softmax with a lazily moved reference point m
+//   O^T += V^T P^T                B = P^T straight from the accumulator registers (the row
+//                                 permutation of the K reads makes them ordered k-slots), A = V^T
+//                                 read from the row-major V tile with the transposing LDS read.
+// The loop is deliberately NOT software pipelined across tiles inside a wavefront: one tile is in
+// flight per wavefront and leading tiles that no query of the workgroup needs masks for run as
+// one straight block.  That keeps the kernel inside 168 registers at head_dim <= 64 (THREE
+// workgroups per CU) and inside 256 above (two), and on this hardware resident wavefronts hide
+// more latency than a deeper pipeline inside one wavefront does: a pipelined variant with twice
+// the registers measured 12 % slower at head_dim 64 and 35-80 % slower at 80 / 128.
+//
+// Reference semantics: slapo/op/attention.py:163-181 (attention_bmk), :97-131 (flash_attn_ref).
+#pragma once
+#include <type_traits>
+
+#include "attn_common.h"
+
+namespace slapo {
+namespace fwd {
+
+constexpr int kWaves = 4;
+constexpr int kThreads = kWaves * 64;
+constexpr int kBM = kWaves * 32;
+constexpr int kBN = 64;
+constexpr float kMaxSlack = 8.0f;  // hysteresis of the softmax reference, log2 units
+
+template <typename T, int DPAD, bool kBias, int kDrop>
+__global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void attn_fwd_kernel(
+    const AttnArgs a) {
+    typedef typename Mma<T>::frag frag_t;
+    typedef TileStage<T, DPAD, kBN, kThreads> Stage;
+    constexpr int kPitch = Stage::kPitch;
+    constexpr int kTileElems = kBN * kPitch;
+    constexpr int DK = DPAD / 16;  // k-steps of S^T = K Q^T
+    constexpr int DV = DPAD / 32;  // 32-row blocks of O^T
+
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    T* k_lds = reinterpret_cast<T*>(smem_raw);  // K[2][tile]
+    T* v_lds = k_lds + 2 * kTileElems;          // V[2][tile]
+
+    const int n_bh = a.batch * a.heads;
+    const int n_qt = (a.sq + kBM - 1) / kBM;
+    const int bh = blockIdx.x % n_bh;
+    const int qt = n_qt - 1 - blockIdx.x / n_bh;  // heaviest (latest) query tiles first
+    const int b = bh / a.heads;
+    const int h = bh % a.heads;
+    const int q0 = qt * kBM;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wavefront-uniform
+    const int g = lane >> 5;
+    const int i_loc = lane & 31;
+    const int wq0 = q0 + wave * 32;  // first query of this wavefront
+    const int q_row = wq0 + i_loc;
+
+    const T* q_base = reinterpret_cast<const T*>(a.q) + b * a.qs[0] + h * a.qs[2];
+    const T* k_base = reinterpret_cast<const T*>(a.k) + b * a.ks[0] + h * a.ks[2];
+    const T* v_base = reinterpret_cast<const T*>(a.v) + b * a.vs[0] + h * a.vs[2];
+
+    int j_lo, j_hi;
+    key_range(a, q0, min(q0 + kBM, a.sq), j_lo, j_hi);
+    if constexpr (kBias)  // skip the tiles that hold nothing but padded keys
+        j_hi = max(j_lo + 1, min(j_hi, padded_key_limit<kThreads>(
+                                           a, b, h, reinterpret_cast<float*>(smem_raw))));
+    const int t_lo = j_lo / kBN;
+    const int t_hi = (j_hi + kBN - 1) / kBN;
+    const int n_tiles = t_hi - t_lo;
+
+    // Start-up loads, all issued before any is used: the Q^T fragments (column i = this lane's
+    // query, k-slots = 8 consecutive head-dim elements) and the first K / V tile.  Addresses are
+    // clamped into the tensors; what was clamped is zeroed afterwards.
+    Stage ks, vs;
+    frag_t qf[DK];
+    {
+        u32x4_t q_raw[DK];
+        const int qr = min(q_row, a.sq - 1);
+#pragma unroll
+        for (int t = 0; t < DK; ++t)
+            q_raw[t] = *reinterpret_cast<const u32x4_t*>(q_base + (int64_t)qr * a.qs[1] +
+                                                         min(16 * t + 8 * g, a.d - 8));
+        ks.load_indexed(k_base, a.ks[1], t_lo * kBN, a.sk, a.d);
+        vs.load_indexed(v_base, a.vs[1], t_lo * kBN, a.sk, a.d);
+#pragma unroll
+        for (int t = 0; t < DK; ++t)
+            qf[t] = __builtin_bit_cast(
+                frag_t, keep_or_zero(q_raw[t], q_row < a.sq && 16 * t + 8 * g < a.d));
+    }
+
+    f32x16_t o_acc[DV];
+#pragma unroll
+    for (int x = 0; x < DV; ++x)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o_acc[x][r] = 0.f;
+    // Without a bias the scores stay in units of the raw dot product and the scale is folded
+    // into the exponential's FMA; with a bias they are converted to log2 units when the bias is
+    // added.  m_run is the reference in score units, m_ref = m_run in log2 units (0 if -inf).
+    float m_run = -INFINITY;
+    float m_ref = 0.f;
+    float l_run = 0.f;  // this lane's share of the running sum
+
+    const int wq_last = min(wq0 + 31, a.sq - 1);
+    const float c_log2 = a.scale_log2;
+    const float slack = kBias ? kMaxSlack : kMaxSlack / c_log2;
+    uint64_t drop_row_base = 0;
+    if constexpr (kDrop != 0)
+        drop_row_base = ((uint64_t)bh * a.sq + (uint64_t)q_row) * (uint64_t)a.sk;
+    const float* bias_row = nullptr;
+    if constexpr (kBias)
+        bias_row = a.bias + b * a.bs[0] + h * a.bs[1] + (int64_t)min(q_row, a.sq - 1) * a.bs[2];
+
+    // per-lane LDS offsets (elements) that do not change from tile to tile
+    const int k_off = pi_row(i_loc) * kPitch + 8 * g;
+    const int v_off = (8 * g + ((lane & 15) >> 2)) * kPitch + ((lane >> 4) & 1) * 16 + 4 * (lane & 3);
+
+    // Wavefront-uniform: does tile t hold any visible key for this wavefront's queries?
+    auto tile_active = [&](int t) __attribute__((always_inline)) {
+        if (wq0 >= a.sq) return false;
+        const int j0 = t * kBN;
+        if (a.causal && j0 > wq_last) return false;
+        if (a.window > 0 && wq0 - (j0 + kBN - 1) >= a.window) return false;
+        return true;
+    };
+    auto tile_needs_mask = [&](int t) __attribute__((always_inline)) {
+        const int j0 = t * kBN;
+        return (j0 + kBN > a.sk) || (a.causal && j0 + kBN - 1 > wq0) ||
+               (a.window > 0 && wq_last - j0 >= a.window);
+    };
+
+    // S^T half = K_half Q^T
+    auto half_scores = [&](const T* kt, int kb, f32x16_t& s) __attribute__((always_inline)) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[r] = 0.f;
+#pragma unroll
+        for (int x = 0; x < DK; ++x)
+            s = Mma<T>::mma32(lds_frag<T>(kt + kb * 32 * kPitch + k_off + 16 * x), qf[x], s);
+    };
+    // bias, masks and maximum of one half; mask_tag: 0 = every key visible, 1 = upper bound only
+    // (causal / key tail), 2 = both bounds (local window).  Returns this lane's maximum.
+    auto finish_half = [&](f32x16_t& s, int t, int kb, auto mask_tag)
+                           __attribute__((always_inline)) -> float {
+        constexpr int kMask = decltype(mask_tag)::value;
+        const int j0 = t * kBN + 32 * kb;
+        // register r is key j0 + 8 g + c with c = acc_row(r, 0); visible iff c_lo <= c <= c_hi
+        int c_lo = 0, c_hi = 0;
+        if constexpr (kMask != 0) {
+            const int k_max = a.causal ? min(a.sk - 1, q_row) : a.sk - 1;
+            c_hi = k_max - j0 - 8 * g;
+            if constexpr (kMask == 2) c_lo = q_row - a.window + 1 - j0 - 8 * g;
+        }
+        float mx = -INFINITY;
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) {
+            if constexpr (kBias) {
+                const int key0 = j0 + acc_row(4 * r4, g);
+                float bv[4] = {0.f, 0.f, 0.f, 0.f};
+                if (a.bias_vec4 && key0 + 3 < a.sk) {
+                    const f32x4_t t4 = *reinterpret_cast<const f32x4_t*>(bias_row + key0);
+                    bv[0] = t4.x, bv[1] = t4.y, bv[2] = t4.z, bv[3] = t4.w;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if (key0 + e < a.sk) bv[e] = bias_row[(int64_t)(key0 + e) * a.bs[3]];
+                }
+#pragma unroll
+                for (int e = 0; e < 4; ++e)
+                    s[4 * r4 + e] = __builtin_fmaf(s[4 * r4 + e], c_log2, bv[e] * kLog2e);
+            }
+            if constexpr (kMask != 0) {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int c = acc_row(4 * r4, 0) + e;
+                    if constexpr (kMask == 2) {
+                        if (c > c_hi || c < c_lo) s[4 * r4 + e] = -INFINITY;
+                    } else {
+                        if (c > c_hi) s[4 * r4 + e] = -INFINITY;
+                    }
+                }
+            }
+            mx = fmaxf(mx, fmaxf(fmaxf(s[4 * r4], s[4 * r4 + 1]),
+                                 fmaxf(s[4 * r4 + 2], s[4 * r4 + 3])));
+        }
+        return mx;
+    };
+    // move the reference point if this tile's maximum calls for it (rare after the first tile)
+    auto update_reference = [&](float mx) __attribute__((always_inline)) {
+        const bool move = (mx > m_run + slack || m_run == -INFINITY) && mx != -INFINITY;
+        if (__builtin_expect(__builtin_amdgcn_ballot_w64(move) != 0, 0)) {
+            const float m_new = move ? mx : m_run;
+            const float m_new_ref = kBias ? m_new : m_new * c_log2;
+            // exp2(old reference - new reference); an unset reference (-inf) scales by 0
+            const float alpha = (m_run == -INFINITY) ? 0.f : fast_exp2(m_ref - m_new_ref);
+            if (move) {
+                m_run = m_new;
+                m_ref = m_new_ref;
+                l_run *= alpha;
+#pragma unroll
+                for (int x = 0; x < DV; ++x)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) o_acc[x][r] *= alpha;
+            }
+        }
+    };
+    // probabilities of one half: exp2, row sum, dropout, pack to T
+    auto half_prob = [&](f32x16_t& s, int t, int kb, uint32_t (&pw)[8])
+                         __attribute__((always_inline)) {
+        float psum = 0.f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            float p;
+            if constexpr (kBias)
+                p = fast_exp2(s[r] - m_ref);
+            else
+                p = fast_exp2(__builtin_fmaf(s[r], c_log2, -m_ref));
+            s[r] = p;
+            psum += p;
+        }
+        l_run += psum;
+        if constexpr (kDrop != 0) {
+            const int j0 = t * kBN + 32 * kb;
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                const int key0 = j0 + acc_row(4 * r4, g);
+                uint32_t bits = 0;
+                if (q_row < a.sq && key0 < a.sk) {
+                    const uint64_t e0 = drop_row_base + (uint64_t)key0;
+                    if constexpr (kDrop == 1)
+                        bits = dropout_keep4_pow2(a.rng, e0 >> 2);
+                    else
+                        bits = dropout_keep_any(a.rng, e0, min(4, a.sk - key0));
+                }
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float p = s[4 * r4 + e];
+                    s[4 * r4 + e] = ((bits >> e) & 1u) ? p * a.rng.inv_keep : 0.f;
+                }
+            }
+        }
+#pragma unroll
+        for (int r2 = 0; r2 < 8; ++r2) pw[r2] = pack2<T>(s[2 * r2], s[2 * r2 + 1]);
+    };
+    // O^T += V_half^T P_half^T
+    auto half_accumulate = [&](const T* vt, int kb, const uint32_t (&pw)[8])
+                               __attribute__((always_inline)) {
+#pragma unroll
+        for (int s2 = 0; s2 < 2; ++s2) {
+            u32x4_t pq = {pw[4 * s2], pw[4 * s2 + 1], pw[4 * s2 + 2], pw[4 * s2 + 3]};
+            const frag_t pf = __builtin_bit_cast(frag_t, pq);
+#pragma unroll
+            for (int x = 0; x < DV; ++x)
+                o_acc[x] = Mma<T>::mma32(
+                    lds_frag_tr<T>(vt + (32 * kb + 16 * s2) * kPitch + v_off + 32 * x, kPitch), pf,
+                    o_acc[x]);
+        }
+    };
+    auto tile_body = [&](const T* kt, const T* vt, int t, auto mask_tag)
+                         __attribute__((always_inline)) {
+        f32x16_t s0, s1;
+        uint32_t pw0[8], pw1[8];
+        half_scores(kt, 0, s0);
+        half_scores(kt, 1, s1);
+        const float mx =
+            max_xor32(fmaxf(finish_half(s0, t, 0, mask_tag), finish_half(s1, t, 1, mask_tag)));
+        update_reference(mx);
+        half_prob(s0, t, 0, pw0);
+        half_accumulate(vt, 0, pw0);
+        half_prob(s1, t, 1, pw1);
+        half_accumulate(vt, 1, pw1);
+    };
+
+    // ---- prologue: tile 0 into LDS ----
+    ks.fix(t_lo * kBN, a.sk, a.d);
+    vs.fix(t_lo * kBN, a.sk, a.d);
+    ks.store(k_lds);
+    vs.store(v_lds);
+    __syncthreads();
+
+    // Iteration r: request tile r+1, process tile r, write tile r+1 into the other slot.
+    // kFast iterations hold tiles that every wavefront of the workgroup sees in full.
+    auto iteration = [&](int r, auto fast_tag) __attribute__((always_inline)) {
+        constexpr bool kFast = decltype(fast_tag)::value;
+        const int t = t_lo + r;
+        const bool have_next = r + 1 < n_tiles;
+        // the next tile is requested unconditionally (rows are clamped into the tensor; after the
+        // last tile the request is wasted) so that it stays straight-line code.  Requesting it
+        // later in the body saves no registers and measures slower.
+        ks.load_indexed(k_base, a.ks[1], (t + 1) * kBN, a.sk, a.d);
+        vs.load_indexed(v_base, a.vs[1], (t + 1) * kBN, a.sk, a.d);
+        const T* kt = k_lds + (r & 1) * kTileElems;
+        const T* vt = v_lds + (r & 1) * kTileElems;
+        if constexpr (kFast) {
+            tile_body(kt, vt, t, std::integral_constant<int, 0>{});
+        } else {
+            if (tile_active(t)) {
+                if (!tile_needs_mask(t))
+                    tile_body(kt, vt, t, std::integral_constant<int, 0>{});
+                else if (a.window > 0)
+                    tile_body(kt, vt, t, std::integral_constant<int, 2>{});
+                else
+                    tile_body(kt, vt, t, std::integral_constant<int, 1>{});
+            }
+        }
+        if (have_next) {
+            ks.fix((t + 1) * kBN, a.sk, a.d);
+            vs.fix((t + 1) * kBN, a.sk, a.d);
+            ks.store(k_lds + ((r + 1) & 1) * kTileElems);
+            vs.store(v_lds + ((r + 1) & 1) * kTileElems);
+        }
+        __syncthreads();
+    };
+    // leading tiles that need neither mask nor activity test for any of the 128 queries
+    int n_fast = 0;
+    if (a.window <= 0 && q0 + kBM <= a.sq) {
+        n_fast = a.sk / kBN;
+        if (a.causal) n_fast = min(n_fast, (q0 + 1) / kBN);
+        n_fast = min(n_fast, n_tiles);
+    }
+    int r = 0;
+    for (; r < n_fast; ++r) iteration(r, std::true_type{});
+    for (; r < n_tiles; ++r) iteration(r, std::false_type{});
+
+    // ---- epilogue ----
+    const float l_tot = sum_xor32(l_run);
+    const float inv_l = 1.0f / l_tot;
+    if (q_row < a.sq) {
+        T* o_row = reinterpret_cast<T*>(a.o) + b * a.os[0] + (int64_t)q_row * a.os[1] + h * a.os[2];
+#pragma unroll
+        for (int x = 0; x < DV; ++x)
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                const int d0 = x * 32 + 8 * r4 + 4 * g;
+                if (d0 < a.d) {
+                    u32x2_t w;
+                    w.x = pack2<T>(o_acc[x][4 * r4 + 0] * inv_l, o_acc[x][4 * r4 + 1] * inv_l);
+                    w.y = pack2<T>(o_acc[x][4 * r4 + 2] * inv_l, o_acc[x][4 * r4 + 3] * inv_l);
+                    *reinterpret_cast<u32x2_t*>(o_row + d0) = w;
+                }
+            }
+        if (g == 0) {
+            const float m_log2 = (m_run == -INFINITY) ? -INFINITY : m_ref;
+            a.lse[(int64_t)bh * a.sq + q_row] = (m_log2 + __builtin_log2f(l_tot)) * kLn2;
+        }
+    }
+}
+
+template <typename T, int DPAD, bool kBias, int kDrop>
+int launch(const AttnArgs& a, hipStream_t st) {
+    typedef TileStage<T, DPAD, kBN, kThreads> Stage;
+    const size_t smem = (size_t)4 * kBN * Stage::kPitch * sizeof(T);
+    const int n_qt = (a.sq + kBM - 1) / kBM;
+    const int64_t blocks = (int64_t)n_qt * a.batch * a.heads;
+    if (blocks <= 0 || blocks > 0x7FFFFFFF) return SLAPO_ERR_SHAPE;
+    auto kern = attn_fwd_kernel<T, DPAD, kBias, kDrop>;
+    if (smem > 48 * 1024) {
+        static bool raised = false;  // per instantiation
+        if (!raised) {
+            if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                    hipFuncAttributeMaxDynamicSharedMemorySize,
+                                    (int)smem) != hipSuccess)
+                return SLAPO_ERR_LAUNCH;
+            raised = true;
+        }
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kThreads), smem, st, a);
+    return check_launch();
+}
+
+template <typename T, int DPAD>
+int dispatch_flags(const AttnArgs& a, hipStream_t st) {
+    if (a.has_bias) {
+        if (a.dropout == 1) return launch<T, DPAD, true, 1>(a, st);
+        if (a.dropout == 2) return launch<T, DPAD, true, 2>(a, st);
+        return launch<T, DPAD, true, 0>(a, st);
+    }
+    if (a.dropout == 1) return launch<T, DPAD, false, 1>(a, st);
+    if (a.dropout == 2) return launch<T, DPAD, false, 2>(a, st);
+    return launch<T, DPAD, false, 0>(a, st);
+}
+
+template <typename T>
+int dispatch(const AttnArgs& a, hipStream_t st) {
+    if (a.d <= 64) return dispatch_flags<T, 64>(a, st);
+    if (a.d <= 96) return dispatch_flags<T, 96>(a, st);
+    if (a.d <= 128) return dispatch_flags<T, 128>(a, st);
+    return SLAPO_ERR_SHAPE;
+}
+
+}  // namespace fwd
+}  // namespace slapo

@@ -135,6 +135,8 @@ def test_compute_entry_points_validate_before_touching_the_device():
     prm.dtype = 2
     prm.q_strides[1] = 68  # rows not 16-byte aligned
     assert lib.slapo_amd_attn_fwd(ctypes.byref(prm), 16, 16, 16, None, 16, 16, None) == -3
+    prm.q_strides[1] = 1 << 24  # row stride beyond the 32-bit tile offsets of the 16-bit kernels
+    assert lib.slapo_amd_attn_fwd(ctypes.byref(prm), 16, 16, 16, None, 16, 16, None) == -2
     prm.q_strides[1] = 64
     prm.p_drop = 0.5  # dropout without a valid plan
     assert lib.slapo_amd_attn_fwd(ctypes.byref(prm), 16, 16, 16, None, 16, 16, None) == -4
