@@ -36,7 +36,7 @@ MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 / bf16
 # WRITE_SIZE (KiB per dispatch), each scaled by the same counter's reading for a 256 MiB copy
 # (FETCH_SIZE reads half the copied bytes: factor 2.0; WRITE_SIZE factor 1.0):
 # (51.55e3 * 2.0 + 49.59e3) KiB.  Summary under profiles/.
-DKDV_TRAFFIC_BYTES = (51.55e3 * 2.0 + 49.59e3) * 1024
+DKDV_TRAFFIC_BYTES = (43.75e3 * 2.0 + 39.58e3) * 1024
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 
 WORKLOAD = dict(name="gpt2-medium causal attention fwd+bwd", dtype="fp16", batch=8, seq=1024,
@@ -285,7 +285,7 @@ def main():
     }
     result["kernels"] = [kern("attn_fwd_kernel<f16, 64, false, 0>", 4 * d * n_pairs, seg_ms[0]),
                          kern("attn_bwd_kernel<f16, 64, false, 0> (dK/dV)", bwd_flops, seg_ms[2]),
-                         kern("attn_bwd_dq_kernel<f16, 64, false, 0>", 6 * d * n_pairs, seg_ms[1])]
+                         kern("attn_bwd_dq_kernel<f16, 64, false, 0, true>", 6 * d * n_pairs, seg_ms[1])]
     if not args.no_epilogues:
         result["epilogue"] = bench_epilogues(device)
     if not args.no_cpu_baseline:
