@@ -25,7 +25,7 @@
 extern "C" {
 #endif
 
-#define SLAPO_AMD_ABI_VERSION 1
+#define SLAPO_AMD_ABI_VERSION 2
 
 /* status codes */
 #define SLAPO_OK 0
@@ -160,7 +160,17 @@ typedef struct slapo_attn_params {
     /* launch plan of the dropout mask over the dense [batch*heads, seqlen_q, seqlen_k] fp32
      * probability tensor (only read when p_drop > 0) */
     slapo_dropout_plan plan;
+    /* Optional (may be NULL), 16-bit types with p_drop > 0 only: device buffer of
+     * slapo_amd_attn_keep_mask_bytes(prm) bytes.  The forward stores the dropout keep bits in it
+     * (one bit per score), and a backward that is given the same buffer reads them instead of
+     * drawing every Philox block again in both of its kernels.  The results are bitwise the
+     * same with and without it.  Layout: uint32 words [batch*heads][ceil(seqlen_k/32)][pitch],
+     * pitch = seqlen_q rounded up to 4; bit j of word (bh, w, i) = keep(query i, key 32 w + j). */
+    void* keep_mask;
 } slapo_attn_params;
+
+/* Size in bytes of the keep_mask buffer (0 when p_drop == 0 or the type is SLAPO_F32). */
+size_t slapo_amd_attn_keep_mask_bytes(const slapo_attn_params* prm);
 
 /* lse: [batch, heads, seqlen_q] fp32, natural-log sum-exp of the masked, scaled scores. */
 int slapo_amd_attn_fwd(const slapo_attn_params* prm, const void* q, const void* k, const void* v,

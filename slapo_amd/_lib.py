@@ -52,6 +52,7 @@ class AttnParams(ctypes.Structure):
         ("o_strides", ctypes.c_int64 * 3),
         ("bias_strides", ctypes.c_int64 * 4),
         ("plan", DropoutPlan),
+        ("keep_mask", ctypes.c_void_p),
     ]
 
 
@@ -103,6 +104,7 @@ PROTOTYPES = {
         ctypes.c_int, [ctypes.POINTER(AttnParams), c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp]
     ),
     "slapo_amd_attn_bwd_workspace_bytes": (ctypes.c_size_t, [ctypes.POINTER(AttnParams)]),
+    "slapo_amd_attn_keep_mask_bytes": (ctypes.c_size_t, [ctypes.POINTER(AttnParams)]),
     "slapo_amd_attn_bwd": (
         ctypes.c_int,
         [ctypes.POINTER(AttnParams), c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp,

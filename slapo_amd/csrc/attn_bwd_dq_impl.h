@@ -75,7 +75,7 @@ __global__ __launch_bounds__(kThreads, (kStagger && DPAD > 64 ? 1 : 2)) void att
     Stage ks, vs;
     // The dropout variants at head_dim 128 have no registers to spare for the tile offsets that
     // `load` keeps: they multiply the addresses out (measured 13 % faster there).
-    constexpr bool kIndexed = kDrop != 0 && DPAD > 96;
+    constexpr bool kIndexed = (kDrop == 1 || kDrop == 2) && DPAD > 96;
     if constexpr (!kIndexed) {
         ks.init(a.ks[1], a.d);
         vs.init(a.vs[1], a.d);
@@ -267,13 +267,25 @@ __global__ __launch_bounds__(kThreads, (kStagger && DPAD > 64 ? 1 : 2)) void att
         }
     };
     // dS^T half = P^T (dP^T - delta), packed to T
-    auto half_ds = [&](const f32x16_t& p, const f32x16_t& dp, int t, int kb, uint32_t (&dw)[8])
-                       __attribute__((always_inline)) {
+    // kDrop == 3: the keep bits of this lane's query for one half of 32 keys, as the forward
+    // stored them (requested at the top of a tile body, used in half_ds)
+    auto mask_word = [&](int t, int kb) __attribute__((always_inline)) -> uint32_t {
+        if constexpr (kDrop == 3) {
+            const int w = min(2 * t + kb, a.mask_words - 1);
+            return a.keep_mask[((int64_t)bh * a.mask_words + w) * a.mask_pitch +
+                               min(q_row, a.sq - 1)];
+        }
+        return 0u;
+    };
+    auto half_ds = [&](const f32x16_t& p, const f32x16_t& dp, int t, int kb, uint32_t mword,
+                       uint32_t (&dw)[8]) __attribute__((always_inline)) {
         const int j0 = t * kBN + kb * 32;
 #pragma unroll
         for (int r4 = 0; r4 < 4; ++r4) {
             uint32_t bits = 0xFu;
-            if constexpr (kDrop != 0) {
+            if constexpr (kDrop == 3) {
+                bits = (mword >> acc_row(4 * r4, g)) & 0xFu;
+            } else if constexpr (kDrop != 0) {
                 const int key0 = j0 + acc_row(4 * r4, g);
                 bits = 0;
                 if (q_row < a.sq && key0 < a.sk) {
@@ -304,25 +316,27 @@ __global__ __launch_bounds__(kThreads, (kStagger && DPAD > 64 ? 1 : 2)) void att
             uint32_t dw0[8];
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb) {
+                const uint32_t mw = mask_word(t, kb);
                 half_s(kt, kb, s0);
                 half_dp(vt, kb, p0);
                 half_exp(s0, t, kb, mask_tag);
-                half_ds(s0, p0, t, kb, dw0);
+                half_ds(s0, p0, t, kb, mw, dw0);
                 half_dq(kt, kb, dw0);
             }
             return;
         }
         f32x16_t s0, s1, p0, p1;
         uint32_t dw0[8], dw1[8];
+        const uint32_t mw0 = mask_word(t, 0), mw1 = mask_word(t, 1);
         half_s(kt, 0, s0);
         half_dp(vt, 0, p0);
         half_exp(s0, t, 0, mask_tag);
         half_s(kt, 1, s1);
-        half_ds(s0, p0, t, 0, dw0);
+        half_ds(s0, p0, t, 0, mw0, dw0);
         half_dp(vt, 1, p1);
         half_exp(s1, t, 1, mask_tag);
         half_dq(kt, 0, dw0);
-        half_ds(s1, p1, t, 1, dw1);
+        half_ds(s1, p1, t, 1, mw1, dw1);
         half_dq(kt, 1, dw1);
     };
 
@@ -365,6 +379,7 @@ __global__ __launch_bounds__(kThreads, (kStagger && DPAD > 64 ? 1 : 2)) void att
                     dq_acc[x] = Mma<T>::mma32(f[s2 * DV + x], df, dq_acc[x]);
             }
         };
+        const uint32_t mw0 = mask_word(t, 0), mw1 = mask_word(t, 1);
         rows(kt, 0, kr0);
         rows(vt, 0, vr0);
         __builtin_amdgcn_sched_barrier(0);
@@ -382,11 +397,11 @@ __global__ __launch_bounds__(kThreads, (kStagger && DPAD > 64 ? 1 : 2)) void att
         cols(1, kq1);
         mma_rows(vr1, gf, p1);
         if constexpr (kDrop == 0) p1 = Mma<T>::mma32(ones_f, ndelta_f, p1);
-        half_ds(s0, p0, t, 0, dw0);
+        half_ds(s0, p0, t, 0, mw0, dw0);
         __builtin_amdgcn_sched_barrier(0);
         mma_cols(kq0, dw0);
         half_exp(s1, t, 1, none);
-        half_ds(s1, p1, t, 1, dw1);
+        half_ds(s1, p1, t, 1, mw1, dw1);
         __builtin_amdgcn_sched_barrier(0);
         mma_cols(kq1, dw1);
     };
@@ -489,10 +504,12 @@ int dispatch_flags(const AttnArgs& a, hipStream_t st) {
     if (a.has_bias) {
         if (a.dropout == 1) return launch<T, DPAD, true, 1, kStagger>(a, st);
         if (a.dropout == 2) return launch<T, DPAD, true, 2, kStagger>(a, st);
+        if (a.dropout == 3) return launch<T, DPAD, true, 3, kStagger>(a, st);
         return launch<T, DPAD, true, 0, kStagger>(a, st);
     }
     if (a.dropout == 1) return launch<T, DPAD, false, 1, kStagger>(a, st);
     if (a.dropout == 2) return launch<T, DPAD, false, 2, kStagger>(a, st);
+    if (a.dropout == 3) return launch<T, DPAD, false, 3, kStagger>(a, st);
     return launch<T, DPAD, false, 0, kStagger>(a, st);
 }
 

@@ -39,7 +39,9 @@ struct BwdSmem {
     static constexpr int kQTile = kBwdBM * kPitch;            // elements
     static constexpr size_t kQBytes = 2 * kQTile * sizeof(T);   // double buffered
     static constexpr size_t kStatBytes = 2 * 2 * kBwdBM * sizeof(float);  // lse, delta; x2 buffers
-    static constexpr size_t kBytes = 2 * kQBytes + kStatBytes;
+    // dropout keep bits of a query tile: one word per wavefront (32 keys) and query; x2 buffers
+    static constexpr size_t kMaskBytes = 2 * kBwdWaves * kBwdBM * sizeof(uint32_t);
+    static constexpr size_t kBytes = 2 * kQBytes + kStatBytes + kMaskBytes;
 };
 
 // KB = blocks of 32 keys per wavefront.  KB = 2 halves the LDS operand traffic per matrix
@@ -48,6 +50,7 @@ struct BwdSmem {
 template <typename T, int DPAD, bool kBias, int kDrop, int KB>
 __global__ __launch_bounds__(kBwdThreads, ((DPAD <= 64 && KB == 1) ? 2 : 1)) void attn_bwd_kernel(
     const AttnArgs a) {
+    static_assert(kDrop != 3 || KB == 1, "the keep-bit tile holds one word per wavefront and query");
     typedef typename Mma<T>::frag frag_t;
     typedef BwdSmem<T, DPAD> SM;
     typedef typename SM::QStage QStage;
@@ -61,6 +64,7 @@ __global__ __launch_bounds__(kBwdThreads, ((DPAD <= 64 && KB == 1) ? 2 : 1)) voi
     T* q_lds = reinterpret_cast<T*>(smem_raw);
     T* g_lds = reinterpret_cast<T*>(smem_raw + SM::kQBytes);
     float* stat_lds = reinterpret_cast<float*>(smem_raw + 2 * SM::kQBytes);
+    uint32_t* mask_lds = reinterpret_cast<uint32_t*>(smem_raw + 2 * SM::kQBytes + SM::kStatBytes);
 
     const int n_bh = a.batch * a.heads;
     const int bh = blockIdx.x % n_bh;
@@ -192,10 +196,26 @@ __global__ __launch_bounds__(kBwdThreads, ((DPAD <= 64 && KB == 1) ? 2 : 1)) voi
         }
     };
 
+    // kDrop == 3: the keep bits that the forward stored.  Thread (w, row) of the workgroup fetches
+    // the word of query row i0 + row for the 32 keys of wavefront w; the tile goes through LDS
+    // like lse / delta.
+    uint32_t mask_reg = 0u;
+    auto load_mask = [&](int i0) __attribute__((always_inline)) {
+        if constexpr (kDrop == 3) {
+            const int w = min((k0 >> 5) + (int)(threadIdx.x >> 6), a.mask_words - 1);
+            const int row = min(i0 + (int)(threadIdx.x & 63), a.mask_pitch - 1);
+            mask_reg = a.keep_mask[((int64_t)bh * a.mask_words + w) * a.mask_pitch + row];
+        }
+    };
+    auto store_mask = [&](int buf) __attribute__((always_inline)) {
+        if constexpr (kDrop == 3) mask_lds[buf * kBwdThreads + threadIdx.x] = mask_reg;
+    };
+
     // rows are clamped into the tensor, so the request is safe even without any query tile
     qst.load(q_base, a.qs[1], t_lo * kBwdBM, a.sq, a.d);
     gst.load(g_base, a.os[1], t_lo * kBwdBM, a.sq, a.d);
     load_stats(t_lo * kBwdBM);
+    load_mask(t_lo * kBwdBM);
 #pragma unroll
     for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
@@ -210,6 +230,7 @@ __global__ __launch_bounds__(kBwdThreads, ((DPAD <= 64 && KB == 1) ? 2 : 1)) voi
         qst.store(q_lds);
         gst.store(g_lds);
         store_stats(0, t_lo * kBwdBM);
+        store_mask(0);
     }
     __syncthreads();
 
@@ -310,8 +331,19 @@ __global__ __launch_bounds__(kBwdThreads, ((DPAD <= 64 && KB == 1) ? 2 : 1)) voi
         }
     };
     // Keep-bits of one key block of a half tile: wq[e] bit 4 * r4 belongs to register 4 * r4 + e.
-    auto keep_bits_half = [&](int kcol, int ih0, uint32_t (&wq)[4]) __attribute__((always_inline)) {
-        if constexpr (kDrop == 1) {
+    // mask_h (kDrop == 3): the words of this wavefront's keys for the 32 queries of the half
+    auto keep_bits_half = [&](int kcol, int ih0, const uint32_t* mask_h, uint32_t (&wq)[4])
+                              __attribute__((always_inline)) {
+        if constexpr (kDrop == 3) {
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                const u32x4_t w = *reinterpret_cast<const u32x4_t*>(mask_h + acc_row(4 * r4, g));
+                wq[0] |= ((w.x >> c_loc) & 1u) << (4 * r4);
+                wq[1] |= ((w.y >> c_loc) & 1u) << (4 * r4);
+                wq[2] |= ((w.z >> c_loc) & 1u) << (4 * r4);
+                wq[3] |= ((w.w >> c_loc) & 1u) << (4 * r4);
+            }
+        } else if constexpr (kDrop == 1) {
             // The four lanes of a quad hold four consecutive keys, i.e. one Philox block per query
             // row.  Lane j of the quad draws the blocks of the rows held in registers j, j+4, j+8,
             // j+12 and the quad exchanges them: 4 blocks per lane instead of 16.
@@ -347,14 +379,14 @@ __global__ __launch_bounds__(kBwdThreads, ((DPAD <= 64 && KB == 1) ? 2 : 1)) voi
     };
     // P (after dropout) and dS = P (dP - delta), packed to T
     auto half_ds = [&](const f32x16_t (&p)[KB], const f32x16_t (&dp)[KB], const float* delta_h,
-                       int ih0, uint32_t (&pw)[KB][8], uint32_t (&dw)[KB][8])
-                       __attribute__((always_inline)) {
+                       const uint32_t* mask_h, int ih0, uint32_t (&pw)[KB][8],
+                       uint32_t (&dw)[KB][8]) __attribute__((always_inline)) {
         uint32_t wq[KB][4];
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) wq[kb][e] = 0u;
-            keep_bits_half(key[kb], ih0, wq[kb]);
+            keep_bits_half(key[kb], ih0, mask_h, wq[kb]);
         }
 #pragma unroll
         for (int r4 = 0; r4 < 4; ++r4) {
@@ -424,6 +456,7 @@ __global__ __launch_bounds__(kBwdThreads, ((DPAD <= 64 && KB == 1) ? 2 : 1)) voi
         const T* gt = g_lds + buf * SM::kQTile;
         const float* lse_t = stat_lds + buf * 2 * kBwdBM;
         const float* delta_t = lse_t + kBwdBM;
+        const uint32_t* mask_t = mask_lds + buf * kBwdThreads + wave * kBwdBM;
         const int i0 = t * kBwdBM;
         const bool have_next = t + 1 < t_hi;
         // The next tile is requested unconditionally (rows are clamped into the tensor; after the
@@ -434,6 +467,7 @@ __global__ __launch_bounds__(kBwdThreads, ((DPAD <= 64 && KB == 1) ? 2 : 1)) voi
             qst.load(q_base, a.qs[1], i0 + kBwdBM, a.sq, a.d);
             gst.load(g_base, a.os[1], i0 + kBwdBM, a.sq, a.d);
             load_stats(i0 + kBwdBM);
+            load_mask(i0 + kBwdBM);
         };
         // (only where two workgroups share a CU and registers are the scarce resource)
         constexpr bool kLateRequest = kFast && DPAD <= 64;
@@ -445,7 +479,7 @@ __global__ __launch_bounds__(kBwdThreads, ((DPAD <= 64 && KB == 1) ? 2 : 1)) voi
             half_sp(qt, gt, lse_t, delta_t, 0, s0, p0);
             half_exp(s0, lse_t, i0, none);
             half_sp(qt, gt, lse_t + 32, delta_t + 32, 1, s1, p1);
-            half_ds(s0, p0, delta_t, i0, pw0, dw0);
+            half_ds(s0, p0, delta_t, mask_t, i0, pw0, dw0);
             half_exp(s1, lse_t + 32, i0 + 32, none);
             if constexpr (kLateRequest) {
                 __builtin_amdgcn_sched_barrier(0);
@@ -453,7 +487,7 @@ __global__ __launch_bounds__(kBwdThreads, ((DPAD <= 64 && KB == 1) ? 2 : 1)) voi
                 __builtin_amdgcn_sched_barrier(0);
             }
             half_out(qt, gt, 0, pw0, dw0);
-            half_ds(s1, p1, delta_t + 32, i0 + 32, pw1, dw1);
+            half_ds(s1, p1, delta_t + 32, mask_t + 32, i0 + 32, pw1, dw1);
             half_out(qt, gt, 1, pw1, dw1);
         } else {
             auto generic_half = [&](int hf) __attribute__((always_inline)) {
@@ -468,7 +502,7 @@ __global__ __launch_bounds__(kBwdThreads, ((DPAD <= 64 && KB == 1) ? 2 : 1)) voi
                     half_exp(s, lse_t + 32 * hf, ih0, std::integral_constant<int, 2>{});
                 else
                     half_exp(s, lse_t + 32 * hf, ih0, std::integral_constant<int, 1>{});
-                half_ds(s, dp, delta_t + 32 * hf, ih0, pw, dw);
+                half_ds(s, dp, delta_t + 32 * hf, mask_t + 32 * hf, ih0, pw, dw);
                 half_out(qt, gt, hf, pw, dw);
             };
             generic_half(0);
@@ -481,6 +515,7 @@ __global__ __launch_bounds__(kBwdThreads, ((DPAD <= 64 && KB == 1) ? 2 : 1)) voi
             qst.store(q_lds + (buf ^ 1) * SM::kQTile);
             gst.store(g_lds + (buf ^ 1) * SM::kQTile);
             store_stats(buf ^ 1, i0 + kBwdBM);
+            store_mask(buf ^ 1);
         }
         __syncthreads();
     };
@@ -559,10 +594,12 @@ int dispatch_flags(const AttnArgs& a, hipStream_t st) {
     if (a.has_bias) {
         if (a.dropout == 1) return launch_kb<T, DPAD, true, 1>(a, st);
         if (a.dropout == 2) return launch_kb<T, DPAD, true, 2>(a, st);
+        if (a.dropout == 3) return launch_kb<T, DPAD, true, 3>(a, st);
         return launch_kb<T, DPAD, true, 0>(a, st);
     }
     if (a.dropout == 1) return launch_kb<T, DPAD, false, 1>(a, st);
     if (a.dropout == 2) return launch_kb<T, DPAD, false, 2>(a, st);
+    if (a.dropout == 3) return launch_kb<T, DPAD, false, 3>(a, st);
     return launch_kb<T, DPAD, false, 0>(a, st);
 }
 

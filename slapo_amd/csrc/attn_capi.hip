@@ -113,7 +113,14 @@ int fill_args(const slapo_attn_params* p, AttnArgs* a, bool backward) {
     } else {
         a->rng = DropoutState{};
     }
-    (void)backward;
+    a->keep_mask = nullptr;
+    a->mask_words = (p->seqlen_k + 31) / 32;
+    a->mask_pitch = (p->seqlen_q + 3) & ~3;
+    if (a->dropout && half && p->keep_mask) {
+        if (!aligned16(p->keep_mask)) return SLAPO_ERR_ALIGN;
+        a->keep_mask = reinterpret_cast<uint32_t*>(p->keep_mask);
+        if (backward) a->dropout = 3;
+    }
     return SLAPO_OK;
 }
 
@@ -134,6 +141,13 @@ bool half_ptrs_ok(std::initializer_list<const void*> ptrs) {
 
 }  // namespace
 
+
+extern "C" size_t slapo_amd_attn_keep_mask_bytes(const slapo_attn_params* p) {
+    if (!p || !(p->p_drop > 0.f) || (p->dtype != SLAPO_F16 && p->dtype != SLAPO_BF16)) return 0;
+    if (p->batch <= 0 || p->heads <= 0 || p->seqlen_q <= 0 || p->seqlen_k <= 0) return 0;
+    const size_t words = (size_t)((p->seqlen_k + 31) / 32) * (size_t)((p->seqlen_q + 3) & ~3);
+    return (size_t)p->batch * p->heads * words * sizeof(uint32_t);
+}
 
 extern "C" int slapo_amd_attn_fwd(const slapo_attn_params* prm, const void* q, const void* k,
                                   const void* v, const float* bias, void* o, float* lse,

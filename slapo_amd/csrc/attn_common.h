@@ -104,6 +104,12 @@ __device__ __forceinline__ void swap32(float v, float& lo_val, float& hi_val) {
     lo_val = a;
     hi_val = b;
 }
+// OR of a value with that of lane l ^ 32
+__device__ __forceinline__ uint32_t or_xor32(uint32_t v) {
+    float a, b;
+    swap32(__builtin_bit_cast(float, v), a, b);
+    return __builtin_bit_cast(uint32_t, a) | __builtin_bit_cast(uint32_t, b);
+}
 __device__ __forceinline__ float max_xor32(float v) {
     float a, b;
     swap32(v, a, b);
@@ -142,8 +148,13 @@ struct AttnArgs {
     int causal, window;
     int has_bias, bias_vec4;  // bias_vec4: s3 == 1, s2 == 0 rows 16B-aligned
     // dropout: 0 = off, 1 = fast mask geometry (plan.vec >= 4, power-of-two thread count and
-    // sk % 4 == 0: one Philox block per aligned group of four keys), 2 = any geometry
+    // sk % 4 == 0: one Philox block per aligned group of four keys), 2 = any geometry,
+    // 3 (backward only) = keep bits read from keep_mask
     int dropout;
+    // Keep bits of the dropout mask, written by the forward when not null: uint32 words
+    // [batch*heads][mask_words][mask_pitch], bit j of word (bh, w, i) = keep(query i, key 32 w + j)
+    uint32_t* keep_mask;
+    int mask_words, mask_pitch;
     float scale, scale_log2;
     DropoutState rng;
 };

@@ -209,7 +209,8 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
         }
     };
     // probabilities of one half: exp2, row sum, dropout, pack to T
-    auto half_prob = [&](f32x16_t& s, int t, int kb, uint32_t (&pw)[8])
+    // (drop_bits: the keep bits of this lane's 16 keys at their position in the half)
+    auto half_prob = [&](f32x16_t& s, int t, int kb, uint32_t (&pw)[8], uint32_t& drop_bits)
                          __attribute__((always_inline)) {
         float psum = 0.f;
 #pragma unroll
@@ -225,6 +226,7 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
         l_run += psum;
         if constexpr (kDrop != 0) {
             const int j0 = t * kBN + 32 * kb;
+            uint32_t mine = 0;  // keep bits of this lane's 16 keys, at their position in the half
 #pragma unroll
             for (int r4 = 0; r4 < 4; ++r4) {
                 const int key0 = j0 + acc_row(4 * r4, g);
@@ -236,12 +238,14 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
                     else
                         bits = dropout_keep_any(a.rng, e0, min(4, a.sk - key0));
                 }
+                mine |= bits << acc_row(4 * r4, g);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const float p = s[4 * r4 + e];
                     s[4 * r4 + e] = ((bits >> e) & 1u) ? p * a.rng.inv_keep : 0.f;
                 }
             }
+            drop_bits = mine;
         }
 #pragma unroll
         for (int r2 = 0; r2 < 8; ++r2) pw[r2] = pack2<T>(s[2 * r2], s[2 * r2 + 1]);
@@ -269,10 +273,26 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
         const float mx =
             max_xor32(fmaxf(finish_half(s0, t, 0, mask_tag), finish_half(s1, t, 1, mask_tag)));
         update_reference(mx);
-        half_prob(s0, t, 0, pw0);
+        uint32_t bits0 = 0, bits1 = 0;
+        half_prob(s0, t, 0, pw0, bits0);
         half_accumulate(vt, 0, pw0);
-        half_prob(s1, t, 1, pw1);
+        half_prob(s1, t, 1, pw1, bits1);
         half_accumulate(vt, 1, pw1);
+        // With dropout and a keep_mask buffer: one word per query and half for the backward.
+        // The (wavefront-uniform) branch sits at the end of the tile, where the basic block ends
+        // anyway; inside the body it would keep the scheduler from mixing the Philox arithmetic
+        // with the matrix instructions (10 % of the forward).
+        if constexpr (kDrop != 0) {
+            if (a.keep_mask != nullptr) {
+                const uint32_t w0 = or_xor32(bits0), w1 = or_xor32(bits1);
+                uint32_t* row = a.keep_mask +
+                                ((int64_t)bh * a.mask_words + 2 * t) * a.mask_pitch + q_row;
+                if (g == 0 && q_row < a.sq) {
+                    if (t * kBN < a.sk) row[0] = w0;
+                    if (t * kBN + 32 < a.sk) row[a.mask_pitch] = w1;
+                }
+            }
+        }
     };
 
     // ---- prologue: tile 0 into LDS ----

@@ -168,7 +168,8 @@ def _usable_layout(t):
     return t
 
 
-def make_attn_params(q, k, v, o, bias, causal, window, scale, p, seed, offset, plan):
+def make_attn_params(q, k, v, o, bias, causal, window, scale, p, seed, offset, plan,
+                     keep_mask=None):
     prm = AttnParams()
     b, sq, h, d = q.shape
     prm.dtype = _lib.dtype_code(q.dtype)
@@ -187,6 +188,8 @@ def make_attn_params(q, k, v, o, bias, causal, window, scale, p, seed, offset, p
         prm.bias_strides = (ctypes.c_int64 * 4)(*bias.stride())
     if plan is not None:
         prm.plan = plan
+    if keep_mask is not None:
+        prm.keep_mask = keep_mask.data_ptr()
     return prm
 
 
@@ -201,22 +204,33 @@ def prepare_bias(attention_mask, b, h, sq, sk):
     return m.expand(b, h, sq, sk)
 
 
-def attn_fwd(q, k, v, bias, causal, window, scale, p, seed, offset, plan):
+def attn_fwd(q, k, v, bias, causal, window, scale, p, seed, offset, plan, save_mask=None):
+    """Returns (o, lse, (q, k, v) as consumed); when save_mask is given (True / False) a fourth
+    item: the dropout keep bits for attn_bwd, or None (save_mask False, p == 0, fp32)."""
     _require_device(q, k, v, bias)
     q, k, v = _usable_layout(q), _usable_layout(k), _usable_layout(v)
     b, sq, h, d = q.shape
     o = torch.empty((b, sq, h, d), dtype=q.dtype, device=q.device)
     lse = torch.empty((b, h, sq), dtype=torch.float32, device=q.device)
     prm = make_attn_params(q, k, v, o, bias, causal, window, scale, p, seed, offset, plan)
+    keep_mask = None
+    if save_mask and o.numel():
+        nbytes = _lib.load().slapo_amd_attn_keep_mask_bytes(ctypes.byref(prm))
+        if nbytes:
+            keep_mask = torch.empty(nbytes // 4, dtype=torch.int32, device=q.device)
+            prm.keep_mask = keep_mask.data_ptr()
     if o.numel():
         with torch.cuda.device(q.device):
             rc = _lib.load().slapo_amd_attn_fwd(ctypes.byref(prm), _ptr(q), _ptr(k), _ptr(v),
                                                 _ptr(bias), _ptr(o), _ptr(lse), _stream())
         _lib.check(rc, "slapo_amd_attn_fwd")
+    if save_mask is not None:
+        return o, lse, (q, k, v), keep_mask
     return o, lse, (q, k, v)
 
 
-def attn_bwd(dout, q, k, v, bias, o, lse, causal, window, scale, p, seed, offset, plan):
+def attn_bwd(dout, q, k, v, bias, o, lse, causal, window, scale, p, seed, offset, plan,
+             keep_mask=None):
     _require_device(dout, q, k, v, o, lse, bias)
     dout = dout if dout.stride() == o.stride() else dout.contiguous()
     if dout.stride() != o.stride():
@@ -224,7 +238,8 @@ def attn_bwd(dout, q, k, v, bias, o, lse, causal, window, scale, p, seed, offset
     dq = torch.empty(q.shape, dtype=q.dtype, device=q.device)
     dk = torch.empty(k.shape, dtype=k.dtype, device=k.device)
     dv = torch.empty(v.shape, dtype=v.dtype, device=v.device)
-    prm = make_attn_params(q, k, v, o, bias, causal, window, scale, p, seed, offset, plan)
+    prm = make_attn_params(q, k, v, o, bias, causal, window, scale, p, seed, offset, plan,
+                           keep_mask)
     if dq.numel() and dk.numel():
         lib = _lib.load()
         nbytes = lib.slapo_amd_attn_bwd_workspace_bytes(ctypes.byref(prm))

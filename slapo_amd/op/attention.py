@@ -45,9 +45,16 @@ def warning_once(msg):
         ATTN_GLOBAL_MSGS.add(msg)
 
 
+# With dropout, the forward hands the keep bits (1 bit per score) to the backward, which then reads
+# them instead of regenerating every Philox block in both of its kernels.  Same gradients, bit
+# for bit; False trades the buffer (B*H*Sq*Sk/8 bytes) for the regeneration.
+SAVE_DROPOUT_MASK = True
+
+
 class _HipAttention(torch.autograd.Function):
-    """Forward saves (q, k, v, bias, out, lse) and the Philox (seed, offset); backward recomputes
-    the probabilities from lse and regenerates the dropout mask -- it never draws."""
+    """Forward saves (q, k, v, bias, out, lse), the Philox (seed, offset) and, with dropout, the
+    keep bits; backward recomputes the probabilities from lse and reads (or regenerates) the
+    dropout mask -- it never draws."""
 
     # pylint: disable=arguments-differ, abstract-method
     @staticmethod
@@ -59,18 +66,19 @@ class _HipAttention(torch.autograd.Function):
             plan = K.dropout_plan(b * h * sq * sk, 4, q.device)
             if p < 1.0:
                 seed, offset = draw_philox(plan.offset_increment, q.device)
-        out, lse, (q, k, v) = K.attn_fwd(q, k, v, bias, causal, window, scale, p, seed, offset,
-                                         plan)
-        ctx.save_for_backward(q, k, v, bias, out, lse)
+        save_mask = SAVE_DROPOUT_MASK and 0.0 < p < 1.0 and any(ctx.needs_input_grad[:3])
+        out, lse, (q, k, v), keep_mask = K.attn_fwd(q, k, v, bias, causal, window, scale, p, seed,
+                                                    offset, plan, save_mask=save_mask)
+        ctx.save_for_backward(q, k, v, bias, out, lse, keep_mask)
         ctx.cfg = (causal, window, scale, p, seed, offset, plan)
         return out
 
     @staticmethod
     def backward(ctx, dout):
-        q, k, v, bias, out, lse = ctx.saved_tensors
+        q, k, v, bias, out, lse, keep_mask = ctx.saved_tensors
         causal, window, scale, p, seed, offset, plan = ctx.cfg
         dq, dk, dv = K.attn_bwd(dout, q, k, v, bias, out, lse, causal, window, scale, p, seed,
-                                offset, plan)
+                                offset, plan, keep_mask)
         return dq, dk, dv, None, None, None, None, None
 
 

@@ -34,7 +34,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_abi_version_and_status_strings():
     lib = _lib.load()
-    assert lib.slapo_amd_abi_version() == 1
+    assert lib.slapo_amd_abi_version() == 2
     assert lib.slapo_amd_status_string(0) == b"ok"
     for code in range(-7, 0):
         assert lib.slapo_amd_status_string(code) not in (b"ok", b"unknown status")
@@ -43,7 +43,7 @@ def test_abi_version_and_status_strings():
 def test_struct_layout_matches_header():
     # sizes the C compiler produces for the two PODs (natural alignment, no packing)
     assert ctypes.sizeof(DropoutPlan) == 32
-    assert ctypes.sizeof(_lib.AttnParams) == 4 * 8 + 2 * 4 + 2 * 8 + 16 * 8 + 32
+    assert ctypes.sizeof(_lib.AttnParams) == 4 * 8 + 2 * 4 + 2 * 8 + 16 * 8 + 32 + 8
 
 
 def test_host_philox_known_answers():
@@ -142,3 +142,10 @@ def test_compute_entry_points_validate_before_touching_the_device():
     assert lib.slapo_amd_attn_fwd(ctypes.byref(prm), 16, 16, 16, None, 16, 16, None) == -4
     prm.p_drop, prm.dtype = 0.0, 1
     assert lib.slapo_amd_attn_bwd_workspace_bytes(ctypes.byref(prm)) == 8 * 4
+    # keep-bit buffer: one uint32 per (batch*head, 32 keys, query rounded up to 4); none without
+    # dropout or for fp32
+    assert lib.slapo_amd_attn_keep_mask_bytes(ctypes.byref(prm)) == 0
+    prm.p_drop, prm.batch, prm.heads, prm.seqlen_q, prm.seqlen_k = 0.1, 2, 3, 70, 65
+    assert lib.slapo_amd_attn_keep_mask_bytes(ctypes.byref(prm)) == 2 * 3 * 3 * 72 * 4
+    prm.dtype = 0
+    assert lib.slapo_amd_attn_keep_mask_bytes(ctypes.byref(prm)) == 0

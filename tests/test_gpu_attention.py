@@ -171,6 +171,70 @@ def test_dropout_mask_bits_read_back_exactly():
     assert max_abs_err(out.cpu().permute(0, 2, 1, 3), keep.double() / (s * (1 - p))) <= 1e-6
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape,causal,window,masked,p", [
+    ((2, 256, 2, 64), True, 0, False, 0.1),     # shift-only mask geometry, staggered kernels
+    ((1, 200, 3, 64), False, 0, True, 0.3),     # ragged tail, padding mask (skipped key tiles)
+    ((1, 131, 2, 32), True, 0, False, 0.5),     # Sk % 4 != 0: per-element mask geometry
+    ((1, 320, 2, 128), True, 0, False, 0.1),    # sequential halves, two workgroups per CU
+    ((1, 320, 2, 128), True, 100, False, 0.1),  # local window (staggered variant at 128)
+    ((1, 192, 2, 80), False, 0, True, 0.2),     # head_dim 80 (padded to 96)
+])
+def test_dropout_keep_bits_saved_by_the_forward(dtype, shape, causal, window, masked, p):
+    """The forward stores the keep bits, the backward reads them: gradients are bitwise those of
+    a backward that regenerates the mask, and the stored bits are torch's own mask."""
+    import ctypes
+
+    from slapo_amd import _lib
+    from slapo_amd.op import _kernels as K
+    from slapo_amd.op import attention as A
+
+    b, s, h, d = shape
+    q, k, v, do, g = _inputs(*shape, dtype)
+    mask = _padding_mask(b, s, dtype, g, s // 3)[0] if masked else None
+    assert A.SAVE_DROPOUT_MASK
+    with_bits = _run(q, k, v, do, mask, causal, window, p)
+    A.SAVE_DROPOUT_MASK = False
+    try:
+        regenerated = _run(q, k, v, do, mask, causal, window, p)
+    finally:
+        A.SAVE_DROPOUT_MASK = True
+    for a, r in zip(with_bits, regenerated):
+        assert torch.equal(a, r)
+
+    # the buffer itself: every word that the forward visits holds torch's mask bits
+    qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
+    plan = K.dropout_plan(b * h * s * s, 4, qd.device)
+    torch.cuda.manual_seed(5)
+    seed, offset = A.draw_philox(plan.offset_increment, qd.device)
+    bias = K.prepare_bias(mask.cuda(), b, h, s, s) if masked else None
+    _, _, _, words = K.attn_fwd(qd, kd, vd, bias, causal, window, d ** -0.5, p, seed, offset, plan,
+                                save_mask=True)
+    prm = K.make_attn_params(qd, kd, vd, qd, None, causal, window, d ** -0.5, p, seed, offset, plan)
+    n_words, pitch = (s + 31) // 32, (s + 3) // 4 * 4
+    assert _lib.load().slapo_amd_attn_keep_mask_bytes(ctypes.byref(prm)) == b * h * n_words * pitch * 4
+    words = words.cpu().view(b * h, n_words, pitch)[:, :, :s].to(torch.int64) & 0xFFFFFFFF
+    bits = ((words.unsqueeze(-1) >> torch.arange(32)) & 1).bool()      # [bh, w, i, 32]
+    got = bits.permute(0, 2, 1, 3).reshape(b * h, s, n_words * 32)[:, :, :s]
+    keep = _torch_keep(b, h, s, s, p)
+    i, j = torch.arange(s)[:, None], torch.arange(s)[None, :]
+    visited = torch.ones(s, s, dtype=torch.bool)
+    if causal:   # the forward skips 64-key tiles above the diagonal of each 32-query group
+        visited &= (j // 64) * 64 <= (i // 32) * 32 + 31
+    if window:   # ... and those wholly outside the window of the group
+        visited &= (i // 32) * 32 - ((j // 64) * 64 + 63) < window
+    if not masked:
+        assert torch.equal(got[:, visited], keep[:, visited])
+    else:  # skipped padded tiles differ per batch: check the unpadded prefix of each batch
+        lens = (mask[:, 0, 0, :] == 0).sum(-1)
+        for bi in range(b):
+            upto = int(lens[bi])
+            sel = visited.clone()
+            sel[:, upto:] = False
+            for hi in range(h):
+                assert torch.equal(got[bi * h + hi][sel], keep[bi * h + hi][sel])
+
+
 def test_strided_views_of_fused_qkv_are_read_in_place():
     b, s, h, d = 2, 160, 4, 64
     g = torch.Generator().manual_seed(1)
