@@ -126,6 +126,39 @@ int slapo_amd_bias_dropout_residual_bwd(const void* grad, void* dx, void* dbias,
                                         uint64_t offset, const slapo_dropout_plan* plan,
                                         void* stream);
 
+/* y = layer_norm(z) * gamma + beta with z = dropout(x + bias, p) + residual over rows of `cols`
+ * elements (biased variance, rstd = 1 / sqrt(var + eps), as torch.nn.LayerNorm); the mask is the
+ * one torch.nn.functional.dropout would draw for the [rows, cols] tensor.  bias and residual may
+ * be NULL.  z is rounded to the tensor type before the statistics are taken, as the unfused
+ * modules do.  Optional outputs for the backward: z [rows, cols], mean and rstd [rows] fp32
+ * (each may be NULL).  Needs cols % (16 / element size) == 0, 16-byte aligned pointers
+ * (SLAPO_ERR_ALIGN) and cols <= 8192 for the 16-bit types, 4096 for fp32 (SLAPO_ERR_SHAPE).
+ * Replaces: the fused module that `.fuse()` builds for the pattern
+ * F.layer_norm(F.dropout(x + bias) + residual) in tests/test_fusion.py:157-204 and
+ * docs/source/scripts/attention-single-gpu.py:333-346. */
+int slapo_amd_bias_dropout_residual_ln_fwd(const void* x, const void* bias, const void* residual,
+                                           const void* gamma, const void* beta, void* z, void* y,
+                                           float* mean, float* rstd, int64_t rows, int64_t cols,
+                                           int dtype, double eps, double p, uint64_t seed,
+                                           uint64_t offset, const slapo_dropout_plan* plan,
+                                           void* stream);
+
+/* Bytes of fp32 workspace the backward below needs when any of dgamma / dbeta / dbias is asked
+ * for: one partial row triple per 16 rows. */
+size_t slapo_amd_ln_bwd_workspace_bytes(int64_t rows, int64_t cols);
+
+/* Backward of slapo_amd_bias_dropout_residual_ln_fwd from grad_y and the saved z, mean, rstd:
+ * dresidual = dz, dx = dz * mask / (1 - p), dgamma / dbeta / dbias = column sums (two-stage, no
+ * atomics).  Every output may be NULL (at least one must not be).  Replaces: autograd of the same
+ * pattern. */
+int slapo_amd_bias_dropout_residual_ln_bwd(const void* grad_y, const void* z, const float* mean,
+                                           const float* rstd, const void* gamma, void* dx,
+                                           void* dresidual, void* dgamma, void* dbeta,
+                                           void* dbias, void* workspace, size_t workspace_bytes,
+                                           int64_t rows, int64_t cols, int dtype, double p,
+                                           uint64_t seed, uint64_t offset,
+                                           const slapo_dropout_plan* plan, void* stream);
+
 /* ------------------------------------------------------------------------------------------
  * Attention:  O = dropout(softmax(Q K^T * scale + bias + mask)) V, forward and backward.
  *

@@ -100,6 +100,18 @@ PROTOTYPES = {
         [c_vp, c_vp, c_vp, c_vp, ctypes.c_size_t, c_i64, c_i64, ctypes.c_int, ctypes.c_double,
          c_u64, c_u64, ctypes.POINTER(DropoutPlan), c_vp],
     ),
+    "slapo_amd_bias_dropout_residual_ln_fwd": (
+        ctypes.c_int,
+        [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, ctypes.c_int,
+         ctypes.c_double, ctypes.c_double, c_u64, c_u64, ctypes.POINTER(DropoutPlan), c_vp],
+    ),
+    "slapo_amd_ln_bwd_workspace_bytes": (ctypes.c_size_t, [c_i64, c_i64]),
+    "slapo_amd_bias_dropout_residual_ln_bwd": (
+        ctypes.c_int,
+        [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, ctypes.c_size_t,
+         c_i64, c_i64, ctypes.c_int, ctypes.c_double, c_u64, c_u64,
+         ctypes.POINTER(DropoutPlan), c_vp],
+    ),
     "slapo_amd_attn_fwd": (
         ctypes.c_int, [ctypes.POINTER(AttnParams), c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp]
     ),

@@ -309,6 +309,273 @@ __global__ __launch_bounds__(256) void colsum_finish_kernel(const float* __restr
 }
 
 // ----------------------------------------------------------------------------------------
+// bias + dropout + residual + LayerNorm (the fusion pattern of tests/test_fusion.py:157-204:
+// layer_norm(dropout(x + bias) + residual)).
+//
+// A row is owned by TPR threads: one wavefront (TPR = 64) up to 64 * V * kLnChunks columns, the
+// whole block (TPR = 256) above, so that every row value stays in registers between the two
+// passes of the statistics and is read from memory once.  z = dropout(x + bias) + residual is
+// rounded to T first and the statistics are taken from the rounded values, i.e. exactly what the
+// unfused modules compute from the stored sum; z is also what the backward reads.
+// ----------------------------------------------------------------------------------------
+constexpr int kLnChunks = 4;         // 16-byte chunks per thread and row (guarded against cols)
+constexpr int kLnRowsPerBlock = 16;  // backward: rows walked by one block (column partial sums)
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+// Sum over the TPR threads of a row.  red: 4 floats of LDS that no other reduction in flight uses
+// (TPR == 256 only; every thread of the block has to call).
+template <int TPR>
+__device__ __forceinline__ float row_sum(float v, float* red) {
+    v = wave_sum(v);
+    if constexpr (TPR == 256) {
+        if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+        __syncthreads();
+        v = (red[0] + red[1]) + (red[2] + red[3]);
+    }
+    return v;
+}
+
+template <typename T, int V, int TPR, int kDrop>
+__global__ __launch_bounds__(256) void bias_dropout_residual_ln_fwd_kernel(
+    const T* __restrict__ x, const T* __restrict__ bias, const T* __restrict__ residual,
+    const T* __restrict__ gamma, const T* __restrict__ beta, T* __restrict__ z_out,
+    T* __restrict__ y, float* __restrict__ mean_out, float* __restrict__ rstd_out, int64_t rows,
+    int cols, float eps, DropoutState s) {
+    constexpr int kRows = 256 / TPR;  // rows per block
+    __shared__ float red[2][4];
+    const int sub = threadIdx.x % TPR;
+    const int64_t row = (int64_t)blockIdx.x * kRows + threadIdx.x / TPR;
+    const bool row_ok = row < rows;  // uniform per wavefront
+    float zf[kLnChunks][V];
+    float sum = 0.f;
+#pragma unroll
+    for (int u = 0; u < kLnChunks; ++u) {
+        const int col0 = (sub + u * TPR) * V;
+#pragma unroll
+        for (int i = 0; i < V; ++i) zf[u][i] = 0.f;
+        if (row_ok && col0 < cols) {
+            const int64_t off = row * cols + col0;
+            const Chunk<T, V> xin = load_chunk<T, V>(x + off);
+            Chunk<T, V> b, r;
+            if (bias) b = load_chunk_cached<T, V>(bias + col0);
+            if (residual) r = load_chunk<T, V>(residual + off);
+            uint32_t bits = 0xFFFFFFFFu;
+            if constexpr (kDrop != 0) bits = keep_bits<V, kDrop>(s, (uint64_t)off);
+            Chunk<T, V> zc;
+#pragma unroll
+            for (int i = 0; i < V; ++i) {
+                float v = Elem<T>::to_f32(xin.v[i]);
+                if (bias) v += Elem<T>::to_f32(b.v[i]);
+                if constexpr (kDrop != 0) v = ((bits >> i) & 1u) ? v * s.inv_keep : 0.0f;
+                if (residual) v += Elem<T>::to_f32(r.v[i]);
+                zc.v[i] = Elem<T>::from_f32(v);
+                zf[u][i] = Elem<T>::to_f32(zc.v[i]);
+                sum += zf[u][i];
+            }
+            if (z_out) store_chunk<T, V>(z_out + off, zc);
+        }
+    }
+    const float inv_n = 1.0f / (float)cols;
+    const float mean = row_sum<TPR>(sum, red[0]) * inv_n;
+    float sq = 0.f;
+#pragma unroll
+    for (int u = 0; u < kLnChunks; ++u) {
+        if ((sub + u * TPR) * V < cols) {
+#pragma unroll
+            for (int i = 0; i < V; ++i) {
+                const float d = zf[u][i] - mean;
+                sq = __builtin_fmaf(d, d, sq);
+            }
+        }
+    }
+    const float var = row_sum<TPR>(sq, red[1]) * inv_n;
+    const float rstd = 1.0f / __builtin_sqrtf(var + eps);
+    if (!row_ok) return;
+#pragma unroll
+    for (int u = 0; u < kLnChunks; ++u) {
+        const int col0 = (sub + u * TPR) * V;
+        if (col0 < cols) {
+            const Chunk<T, V> g = load_chunk_cached<T, V>(gamma + col0);
+            const Chunk<T, V> be = load_chunk_cached<T, V>(beta + col0);
+            Chunk<T, V> o;
+#pragma unroll
+            for (int i = 0; i < V; ++i)
+                o.v[i] = Elem<T>::from_f32(__builtin_fmaf((zf[u][i] - mean) * rstd,
+                                                          Elem<T>::to_f32(g.v[i]),
+                                                          Elem<T>::to_f32(be.v[i])));
+            store_chunk<T, V>(y + row * cols + col0, o);
+        }
+    }
+    if (sub == 0) {
+        if (mean_out) mean_out[row] = mean;
+        if (rstd_out) rstd_out[row] = rstd;
+    }
+}
+
+// Backward of the above.  With xh = (z - mean) rstd and g = dy gamma:
+//   dz = rstd (g - mean_c(g) - xh mean_c(g xh)),  dresidual = dz,  dx = dz keep / (1 - p),
+//   dgamma = sum_r dy xh,  dbeta = sum_r dy,  dbias = sum_r dx.
+// A block walks kLnRowsPerBlock rows and keeps the three column sums of its threads in
+// registers; they leave as one fp32 partial row triple per block ([block][3][cols]: dgamma, dbeta,
+// dbias) for ln_finish_kernel.  No atomics: the result does not depend on scheduling.
+template <typename T, int V, int TPR, int kDrop>
+__global__ __launch_bounds__(256) void bias_dropout_residual_ln_bwd_kernel(
+    const T* __restrict__ dy, const T* __restrict__ z, const float* __restrict__ mean,
+    const float* __restrict__ rstd, const T* __restrict__ gamma, T* __restrict__ dx,
+    T* __restrict__ dres, float* __restrict__ partial, int64_t rows, int cols, DropoutState s) {
+    constexpr int kRows = 256 / TPR;  // rows in flight per block
+    constexpr int kIters = kLnRowsPerBlock / kRows;
+    constexpr int kCombCols = TPR == 64 ? 64 * V * kLnChunks : 1;
+    __shared__ float red[2][2][4];
+    __shared__ float comb[3 * kCombCols];
+    const int sub = threadIdx.x % TPR;
+    const int rr = threadIdx.x / TPR;
+    Chunk<T, V> gm[kLnChunks];
+    float acc_g[kLnChunks][V], acc_b[kLnChunks][V], acc_x[kLnChunks][V];
+#pragma unroll
+    for (int u = 0; u < kLnChunks; ++u) {
+        const int col0 = (sub + u * TPR) * V;
+        if (col0 < cols) gm[u] = load_chunk_cached<T, V>(gamma + col0);
+#pragma unroll
+        for (int i = 0; i < V; ++i) acc_g[u][i] = 0.f, acc_b[u][i] = 0.f, acc_x[u][i] = 0.f;
+    }
+    const float inv_n = 1.0f / (float)cols;
+#pragma unroll 1
+    for (int it = 0; it < kIters; ++it) {
+        const int64_t row = (int64_t)blockIdx.x * kLnRowsPerBlock + it * kRows + rr;
+        const bool row_ok = row < rows;  // uniform per wavefront
+        Chunk<T, V> gy[kLnChunks], zz[kLnChunks];
+        float m = 0.f, rs = 0.f, s1 = 0.f, s2 = 0.f;
+        if (row_ok) {
+            m = mean[row];
+            rs = rstd[row];
+        }
+#pragma unroll
+        for (int u = 0; u < kLnChunks; ++u) {
+            const int col0 = (sub + u * TPR) * V;
+            if (row_ok && col0 < cols) {
+                const int64_t off = row * cols + col0;
+                gy[u] = load_chunk<T, V>(dy + off);
+                zz[u] = load_chunk<T, V>(z + off);
+#pragma unroll
+                for (int i = 0; i < V; ++i) {
+                    const float d = Elem<T>::to_f32(gy[u].v[i]);
+                    const float xh = (Elem<T>::to_f32(zz[u].v[i]) - m) * rs;
+                    const float g = d * Elem<T>::to_f32(gm[u].v[i]);
+                    s1 += g;
+                    s2 = __builtin_fmaf(g, xh, s2);
+                    acc_g[u][i] = __builtin_fmaf(d, xh, acc_g[u][i]);
+                    acc_b[u][i] += d;
+                }
+            }
+        }
+        const float c1 = row_sum<TPR>(s1, red[it & 1][0]) * inv_n;
+        const float c2 = row_sum<TPR>(s2, red[it & 1][1]) * inv_n;
+#pragma unroll
+        for (int u = 0; u < kLnChunks; ++u) {
+            const int col0 = (sub + u * TPR) * V;
+            if (row_ok && col0 < cols) {
+                const int64_t off = row * cols + col0;
+                uint32_t bits = 0xFFFFFFFFu;
+                if constexpr (kDrop != 0) bits = keep_bits<V, kDrop>(s, (uint64_t)off);
+                Chunk<T, V> oz, ox;
+#pragma unroll
+                for (int i = 0; i < V; ++i) {
+                    const float xh = (Elem<T>::to_f32(zz[u].v[i]) - m) * rs;
+                    const float g = Elem<T>::to_f32(gy[u].v[i]) * Elem<T>::to_f32(gm[u].v[i]);
+                    const float dz = rs * (g - c1 - xh * c2);
+                    float d = dz;
+                    if constexpr (kDrop != 0) d = ((bits >> i) & 1u) ? dz * s.inv_keep : 0.0f;
+                    oz.v[i] = Elem<T>::from_f32(dz);
+                    ox.v[i] = Elem<T>::from_f32(d);
+                    acc_x[u][i] += d;
+                }
+                if (dres) store_chunk<T, V>(dres + off, oz);
+                if (dx) store_chunk<T, V>(dx + off, ox);
+            }
+        }
+    }
+    if (!partial) return;
+    float* out = partial + (int64_t)blockIdx.x * 3 * cols;
+    if constexpr (TPR == 256) {
+#pragma unroll
+        for (int u = 0; u < kLnChunks; ++u) {
+            const int col0 = (sub + u * TPR) * V;
+            if (col0 < cols) {
+#pragma unroll
+                for (int i = 0; i < V; ++i) {
+                    out[col0 + i] = acc_g[u][i];
+                    out[cols + col0 + i] = acc_b[u][i];
+                    out[2 * cols + col0 + i] = acc_x[u][i];
+                }
+            }
+        }
+    } else {
+        // the four wavefronts (row groups) add their sums in turn, then the block writes them
+#pragma unroll 1
+        for (int k = 0; k < kRows; ++k) {
+            if (rr == k) {
+#pragma unroll
+                for (int u = 0; u < kLnChunks; ++u) {
+                    const int col0 = (sub + u * TPR) * V;
+                    if (col0 < cols) {
+#pragma unroll
+                        for (int i = 0; i < V; ++i) {
+                            const int c = col0 + i;
+                            comb[c] = (k ? comb[c] : 0.f) + acc_g[u][i];
+                            comb[cols + c] = (k ? comb[cols + c] : 0.f) + acc_b[u][i];
+                            comb[2 * cols + c] = (k ? comb[2 * cols + c] : 0.f) + acc_x[u][i];
+                        }
+                    }
+                }
+            }
+            __syncthreads();
+        }
+        for (int c = threadIdx.x; c < 3 * cols; c += 256) out[c] = comb[c];
+    }
+}
+
+// Second stage: partial is [n_partials][3 * cols]; column c of it belongs to dgamma (c < cols),
+// dbeta or dbias.  Same shape of work as colsum_finish_kernel.
+template <typename T>
+__global__ __launch_bounds__(256) void ln_finish_kernel(const float* __restrict__ partial,
+                                                        T* __restrict__ dgamma,
+                                                        T* __restrict__ dbeta,
+                                                        T* __restrict__ dbias, int64_t n_partials,
+                                                        int cols) {
+    __shared__ float red[kFinRows][kFinCols + 1];
+    const int cx = threadIdx.x % kFinCols;
+    const int ry = threadIdx.x / kFinCols;
+    const int64_t cols3 = 3 * (int64_t)cols;
+    const int64_t c = (int64_t)blockIdx.x * kFinCols + cx;
+    float t = 0.f;
+    if (c < cols3) {
+        float t0 = 0.f, t1 = 0.f;
+        int64_t k = ry;
+        for (; k + kFinRows < n_partials; k += 2 * kFinRows) {
+            t0 += partial[k * cols3 + c];
+            t1 += partial[(k + kFinRows) * cols3 + c];
+        }
+        for (; k < n_partials; k += kFinRows) t0 += partial[k * cols3 + c];
+        t = t0 + t1;
+    }
+    red[ry][cx] = t;
+    __syncthreads();
+    if (ry == 0 && c < cols3) {
+        float sum = 0.f;
+#pragma unroll
+        for (int r = 0; r < kFinRows; ++r) sum += red[r][cx];
+        const int which = (int)(c / cols);
+        T* dst = which == 0 ? dgamma : which == 1 ? dbeta : dbias;
+        if (dst) dst[c - (int64_t)which * cols] = Elem<T>::from_f32(sum);
+    }
+}
+
+// ----------------------------------------------------------------------------------------
 // Host dispatch
 // ----------------------------------------------------------------------------------------
 struct RowGeom {
@@ -469,6 +736,84 @@ int dropres_bwd_dispatch(const void* grad, void* dx, void* dbias, void* ws, int6
     return finish_colsum<T>((const float*)ws, dbias, rows, cols, st);
 }
 
+template <typename T>
+inline int ln_geometry(int64_t rows, int64_t cols, bool* wide) {
+    constexpr int V = Elem<T>::kPerVec;
+    if (cols % V != 0) return SLAPO_ERR_ALIGN;
+    if (cols > 256 * V * kLnChunks) return SLAPO_ERR_SHAPE;
+    *wide = cols > 64 * V * kLnChunks;
+    if (rows > 0x7FFFFFFF) return SLAPO_ERR_SHAPE;
+    return SLAPO_OK;
+}
+
+template <typename T>
+int ln_fwd_dispatch(const void* x, const void* bias, const void* residual, const void* gamma,
+                    const void* beta, void* z, void* y, float* mean, float* rstd, int64_t rows,
+                    int64_t cols, float eps, bool dropout, const DropoutState& s,
+                    hipStream_t st) {
+    constexpr int V = Elem<T>::kPerVec;
+    bool wide = false;
+    int rc = ln_geometry<T>(rows, cols, &wide);
+    if (rc != SLAPO_OK) return rc;
+    for (const void* p : {x, bias, residual, gamma, beta, (const void*)z, (const void*)y})
+        if (p && !aligned16(p)) return SLAPO_ERR_ALIGN;
+    const int mode = !dropout ? 0 : (s.g_shift >= 0 && s.t_shift >= 0) ? 1 : 2;
+#define SLAPO_LAUNCH_LN(TPR, MODE)                                                              \
+    hipLaunchKernelGGL((bias_dropout_residual_ln_fwd_kernel<T, V, TPR, MODE>),                  \
+                       dim3((unsigned)((rows + (256 / TPR) - 1) / (256 / TPR))), dim3(256), 0,  \
+                       st, (const T*)x, (const T*)bias, (const T*)residual, (const T*)gamma,    \
+                       (const T*)beta, (T*)z, (T*)y, mean, rstd, rows, (int)cols, eps, s)
+    if (wide) {
+        if (mode == 0) SLAPO_LAUNCH_LN(256, 0);
+        if (mode == 1) SLAPO_LAUNCH_LN(256, 1);
+        if (mode == 2) SLAPO_LAUNCH_LN(256, 2);
+    } else {
+        if (mode == 0) SLAPO_LAUNCH_LN(64, 0);
+        if (mode == 1) SLAPO_LAUNCH_LN(64, 1);
+        if (mode == 2) SLAPO_LAUNCH_LN(64, 2);
+    }
+#undef SLAPO_LAUNCH_LN
+    return check_launch();
+}
+
+template <typename T>
+int ln_bwd_dispatch(const void* dy, const void* z, const float* mean, const float* rstd,
+                    const void* gamma, void* dx, void* dres, void* dgamma, void* dbeta,
+                    void* dbias, void* ws, int64_t rows, int64_t cols, bool dropout,
+                    const DropoutState& s, hipStream_t st) {
+    constexpr int V = Elem<T>::kPerVec;
+    bool wide = false;
+    int rc = ln_geometry<T>(rows, cols, &wide);
+    if (rc != SLAPO_OK) return rc;
+    for (const void* p : {dy, z, gamma, (const void*)dx, (const void*)dres})
+        if (p && !aligned16(p)) return SLAPO_ERR_ALIGN;
+    const bool want_sums = dgamma || dbeta || dbias;
+    const int64_t n_blocks = (rows + kLnRowsPerBlock - 1) / kLnRowsPerBlock;
+    float* partial = want_sums ? (float*)ws : nullptr;
+    const int mode = !dropout ? 0 : (s.g_shift >= 0 && s.t_shift >= 0) ? 1 : 2;
+#define SLAPO_LAUNCH_LNB(TPR, MODE)                                                             \
+    hipLaunchKernelGGL((bias_dropout_residual_ln_bwd_kernel<T, V, TPR, MODE>),                  \
+                       dim3((unsigned)n_blocks), dim3(256), 0, st, (const T*)dy, (const T*)z,   \
+                       mean, rstd, (const T*)gamma, (T*)dx, (T*)dres, partial, rows, (int)cols, \
+                       s)
+    if (wide) {
+        if (mode == 0) SLAPO_LAUNCH_LNB(256, 0);
+        if (mode == 1) SLAPO_LAUNCH_LNB(256, 1);
+        if (mode == 2) SLAPO_LAUNCH_LNB(256, 2);
+    } else {
+        if (mode == 0) SLAPO_LAUNCH_LNB(64, 0);
+        if (mode == 1) SLAPO_LAUNCH_LNB(64, 1);
+        if (mode == 2) SLAPO_LAUNCH_LNB(64, 2);
+    }
+#undef SLAPO_LAUNCH_LNB
+    rc = check_launch();
+    if (rc != SLAPO_OK || !want_sums) return rc;
+    const unsigned blocks = (unsigned)((3 * cols + kFinCols - 1) / kFinCols);
+    hipLaunchKernelGGL((ln_finish_kernel<T>), dim3(blocks), dim3(256), 0, st, partial,
+                       (T*)dgamma, (T*)dbeta, (T*)dbias, n_blocks, (int)cols);
+    return check_launch();
+}
+
 inline bool dims_ok(int64_t rows, int64_t cols) {
     return rows > 0 && cols > 0 && rows <= (int64_t)1 << 40 && cols <= (int64_t)1 << 30;
 }
@@ -551,6 +896,60 @@ extern "C" int slapo_amd_bias_dropout_residual_bwd(const void* grad, void* dx, v
     }
     hipStream_t st = (hipStream_t)stream;
 #define CALL(T) dropres_bwd_dispatch<T>(grad, dx, dbias, workspace, rows, cols, dropout, s, st)
+    SLAPO_DISPATCH_DTYPE(dtype, CALL)
+#undef CALL
+}
+
+extern "C" size_t slapo_amd_ln_bwd_workspace_bytes(int64_t rows, int64_t cols) {
+    if (rows <= 0 || cols <= 0) return 0;
+    const int64_t n_blocks = (rows + kLnRowsPerBlock - 1) / kLnRowsPerBlock;
+    return (size_t)n_blocks * 3 * (size_t)cols * sizeof(float);
+}
+
+extern "C" int slapo_amd_bias_dropout_residual_ln_fwd(
+    const void* x, const void* bias, const void* residual, const void* gamma, const void* beta,
+    void* z, void* y, float* mean, float* rstd, int64_t rows, int64_t cols, int dtype,
+    double eps, double p, uint64_t seed, uint64_t offset, const slapo_dropout_plan* plan,
+    void* stream) {
+    if (!x || !gamma || !beta || !y) return SLAPO_ERR_ARG;
+    if (!dims_ok(rows, cols)) return SLAPO_ERR_SHAPE;
+    if (!(p >= 0.0 && p <= 1.0) || !(eps >= 0.0)) return SLAPO_ERR_ARG;
+    const bool dropout = p > 0.0;
+    DropoutState s = {};
+    if (dropout) {
+        if (!plan_ok(plan, rows * cols)) return SLAPO_ERR_ARG;
+        s = make_dropout_state(*plan, p, seed, offset);
+    }
+    hipStream_t st = (hipStream_t)stream;
+#define CALL(T)                                                                                \
+    ln_fwd_dispatch<T>(x, bias, residual, gamma, beta, z, y, mean, rstd, rows, cols, (float)eps, \
+                       dropout, s, st)
+    SLAPO_DISPATCH_DTYPE(dtype, CALL)
+#undef CALL
+}
+
+extern "C" int slapo_amd_bias_dropout_residual_ln_bwd(
+    const void* grad_y, const void* z, const float* mean, const float* rstd, const void* gamma,
+    void* dx, void* dresidual, void* dgamma, void* dbeta, void* dbias, void* workspace,
+    size_t workspace_bytes, int64_t rows, int64_t cols, int dtype, double p, uint64_t seed,
+    uint64_t offset, const slapo_dropout_plan* plan, void* stream) {
+    if (!grad_y || !z || !mean || !rstd || !gamma) return SLAPO_ERR_ARG;
+    if (!dx && !dresidual && !dgamma && !dbeta && !dbias) return SLAPO_ERR_ARG;
+    if (!dims_ok(rows, cols)) return SLAPO_ERR_SHAPE;
+    if (!(p >= 0.0 && p <= 1.0)) return SLAPO_ERR_ARG;
+    if ((dgamma || dbeta || dbias) &&
+        (!workspace || workspace_bytes < slapo_amd_ln_bwd_workspace_bytes(rows, cols)))
+        return SLAPO_ERR_WORKSPACE;
+    const bool dropout = p > 0.0;
+    DropoutState s = {};
+    if (dropout) {
+        if (!plan_ok(plan, rows * cols)) return SLAPO_ERR_ARG;
+        s = make_dropout_state(*plan, p, seed, offset);
+    }
+    hipStream_t st = (hipStream_t)stream;
+#define CALL(T)                                                                               \
+    ln_bwd_dispatch<T>(grad_y, z, mean, rstd, gamma, dx, dresidual, dgamma, dbeta, dbias,    \
+                       workspace, rows, cols, dropout, s, st)
     SLAPO_DISPATCH_DTYPE(dtype, CALL)
 #undef CALL
 }

@@ -1,7 +1,9 @@
 """Fused ops with the reference's names (slapo/op/__init__.py:4-8) on HIP kernels."""
 from .attention import FlashAttention, FlashAttentionOp, hip_attention
-from .fused_bias import (BiasGeLUFunction, HipBiasDropoutResidual, HipBiasGeLU, bias_dropout,
-                         bias_dropout_residual, bias_gelu, bias_new_gelu)
+from .fused_bias import (BiasGeLUFunction, HipBiasDropoutResidual,
+                         HipBiasDropoutResidualLayerNorm, HipBiasGeLU, bias_dropout,
+                         bias_dropout_residual, bias_dropout_residual_layer_norm, bias_gelu,
+                         bias_new_gelu)
 from .linear import (FusedQKV, LinearWithAct, LinearWithDropout, LinearWithSeparateBias,
                      LinearWithSyncFunc)
 from .mlp import FusedMLP

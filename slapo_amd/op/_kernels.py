@@ -136,6 +136,73 @@ def bias_dropout_residual_bwd(grad, bias_like, p, seed, offset, plan, need_dx=Tr
     return dx, dbias
 
 
+def bias_dropout_residual_ln_fwd(x, bias, residual, weight, ln_bias, eps, p, seed, offset, plan,
+                                 save_for_backward=True):
+    """Returns (y, z, mean, rstd); the last three are None without save_for_backward."""
+    _require_device(x, bias, residual, weight, ln_bias)
+    x = x.contiguous()
+    bias, residual, weight, ln_bias = _same_dtype(
+        x, bias.contiguous() if bias is not None else None,
+        residual.contiguous() if residual is not None else None, weight.contiguous(),
+        ln_bias.contiguous())
+    if residual is not None and residual.shape != x.shape:
+        raise ValueError("residual must have the shape of x")
+    cols = x.shape[-1]
+    if weight.shape != (cols,) or ln_bias.shape != (cols,) or (
+            bias is not None and bias.shape != (cols,)):
+        raise ValueError("bias, weight and ln_bias must be 1-D of the last dimension of x")
+    rows = x.numel() // max(cols, 1)
+    y = torch.empty_like(x)
+    z = mean = rstd = None
+    if save_for_backward:
+        z = torch.empty_like(x)
+        mean = torch.empty(rows, dtype=torch.float32, device=x.device)
+        rstd = torch.empty(rows, dtype=torch.float32, device=x.device)
+    if x.numel() == 0:
+        return y, z, mean, rstd
+    with torch.cuda.device(x.device):
+        rc = _lib.load().slapo_amd_bias_dropout_residual_ln_fwd(
+            _ptr(x), _ptr(bias), _ptr(residual), _ptr(weight), _ptr(ln_bias), _ptr(z), _ptr(y),
+            _ptr(mean), _ptr(rstd), rows, cols, _lib.dtype_code(x.dtype), float(eps), float(p),
+            seed, offset, ctypes.byref(plan) if plan is not None else None, _stream())
+    _lib.check(rc, "slapo_amd_bias_dropout_residual_ln_fwd")
+    return y, z, mean, rstd
+
+
+def bias_dropout_residual_ln_bwd(grad, z, mean, rstd, weight, p, seed, offset, plan, need_dx=True,
+                                 need_dres=True, need_dweight=True, need_dln_bias=True,
+                                 need_dbias=True):
+    """Returns (dx, dresidual, dweight, dln_bias, dbias); entries not asked for are None."""
+    _require_device(grad, z, mean, rstd, weight)
+    grad = grad.contiguous()
+    (weight,) = _same_dtype(z, weight.contiguous())
+    cols = z.shape[-1]
+    rows = z.numel() // max(cols, 1)
+    vec = lambda need: torch.empty(cols, dtype=z.dtype, device=z.device) if need else None
+    dx = torch.empty_like(z) if need_dx else None
+    dres = torch.empty_like(z) if need_dres else None
+    dw, dlb, db = vec(need_dweight), vec(need_dln_bias), vec(need_dbias)
+    outs = (dx, dres, dw, dlb, db)
+    if z.numel() == 0 or all(o is None for o in outs):
+        for o in (dw, dlb, db):
+            if o is not None:
+                o.zero_()
+        return outs
+    lib = _lib.load()
+    with torch.cuda.device(z.device):
+        ws, nbytes = None, 0
+        if need_dweight or need_dln_bias or need_dbias:
+            nbytes = lib.slapo_amd_ln_bwd_workspace_bytes(rows, cols)
+            ws = torch.empty(max(nbytes // 4, 1), dtype=torch.float32, device=z.device)
+        rc = lib.slapo_amd_bias_dropout_residual_ln_bwd(
+            _ptr(grad), _ptr(z), _ptr(mean), _ptr(rstd), _ptr(weight), _ptr(dx), _ptr(dres),
+            _ptr(dw), _ptr(dlb), _ptr(db), _ptr(ws), nbytes, rows, cols,
+            _lib.dtype_code(z.dtype), float(p), seed, offset,
+            ctypes.byref(plan) if plan is not None else None, _stream())
+    _lib.check(rc, "slapo_amd_bias_dropout_residual_ln_bwd")
+    return outs
+
+
 def dropout_mask(numel, elem_bytes, p, seed, offset, device):
     """Boolean keep-mask [numel] drawn on the device (debugging / test aid)."""
     plan = dropout_plan(numel, elem_bytes, device)

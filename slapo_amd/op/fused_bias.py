@@ -91,6 +91,49 @@ def bias_dropout_residual(x: torch.Tensor, bias: torch.Tensor, residual: torch.T
     return _BiasDropoutResidual.apply(x, bias, residual, float(p) if training else 0.0)
 
 
+class _BiasDropoutResidualLayerNorm(torch.autograd.Function):
+    # pylint: disable=arguments-differ, abstract-method
+    @staticmethod
+    def forward(ctx, x, bias, residual, weight, ln_bias, p, eps):
+        plan, seed, offset = None, 0, 0
+        if 0.0 < p:
+            plan = K.dropout_plan(x.numel(), x.element_size(), x.device)
+            if p < 1.0:
+                # The generator moves exactly as it would for F.dropout on this tensor.
+                seed, offset = draw_philox(plan.offset_increment, x.device)
+        need_grad = any(ctx.needs_input_grad[:5])
+        y, z, mean, rstd = K.bias_dropout_residual_ln_fwd(
+            x, bias, residual, weight, ln_bias, eps, p, seed, offset, plan,
+            save_for_backward=need_grad)
+        ctx.cfg = (p, seed, offset, plan, bias is not None, residual is not None)
+        ctx.dtypes = tuple(t.dtype if t is not None else None for t in (bias, weight, ln_bias))
+        ctx.save_for_backward(z, mean, rstd, weight)
+        return y
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        z, mean, rstd, weight = ctx.saved_tensors
+        p, seed, offset, plan, has_bias, has_residual = ctx.cfg
+        need = ctx.needs_input_grad
+        dx, dres, dw, dlb, db = K.bias_dropout_residual_ln_bwd(
+            grad_output, z, mean, rstd, weight, p, seed, offset, plan, need_dx=need[0],
+            need_dres=has_residual and need[2], need_dweight=need[3], need_dln_bias=need[4],
+            need_dbias=has_bias and need[1])
+        cast = lambda t, dt: t if t is None or t.dtype == dt else t.to(dt)
+        return (dx, cast(db, ctx.dtypes[0]), dres, cast(dw, ctx.dtypes[1]),
+                cast(dlb, ctx.dtypes[2]), None, None)
+
+
+def bias_dropout_residual_layer_norm(x: torch.Tensor, bias, residual, weight: torch.Tensor,
+                                     ln_bias: torch.Tensor, p: float = 0.5, eps: float = 1e-5,
+                                     training: bool = True) -> torch.Tensor:
+    """layer_norm(dropout(x + bias) + residual) over the last dimension, the pattern of
+    tests/test_fusion.py:184-185 (bias and residual may be None)."""
+    _check_p(p)
+    return _BiasDropoutResidualLayerNorm.apply(x, bias, residual, weight, ln_bias,
+                                               float(p) if training else 0.0, float(eps))
+
+
 def _check_p(p):
     if p < 0.0 or p > 1.0:
         raise ValueError(f"dropout probability has to be between 0 and 1, but got {p}")
@@ -116,3 +159,37 @@ class HipBiasDropoutResidual(nn.Module):
 
     def extra_repr(self):
         return f"p={self.p}"
+
+
+class HipBiasDropoutResidualLayerNorm(nn.Module):
+    """Replacement payload for a matched `layer_norm(dropout(x + bias) + residual)` subgraph;
+    owns the LayerNorm parameters under the names of `nn.LayerNorm` (`weight`, `bias`)."""
+
+    def __init__(self, normalized_shape: int, p: float = 0.5, eps: float = 1e-5, device=None,
+                 dtype=None):
+        super().__init__()
+        _check_p(p)
+        if not isinstance(normalized_shape, int):
+            if len(normalized_shape) != 1:
+                raise NotImplementedError("only the last dimension can be normalized")
+            normalized_shape = int(normalized_shape[0])
+        self.normalized_shape = (normalized_shape,)
+        self.p, self.eps = p, eps
+        self.weight = nn.Parameter(torch.ones(normalized_shape, device=device, dtype=dtype))
+        self.bias = nn.Parameter(torch.zeros(normalized_shape, device=device, dtype=dtype))
+
+    @classmethod
+    def from_layer_norm(cls, ln: nn.LayerNorm, p: float):
+        """Takes over the parameters of an existing nn.LayerNorm (shared, not copied)."""
+        if not ln.elementwise_affine or ln.bias is None:
+            raise NotImplementedError("LayerNorm without affine parameters")
+        mod = cls(ln.normalized_shape, p, ln.eps, device=ln.weight.device, dtype=ln.weight.dtype)
+        mod.weight, mod.bias = ln.weight, ln.bias
+        return mod
+
+    def forward(self, x, bias, residual):
+        return bias_dropout_residual_layer_norm(x, bias, residual, self.weight, self.bias,
+                                                self.p, self.eps, self.training)
+
+    def extra_repr(self):
+        return f"{self.normalized_shape}, p={self.p}, eps={self.eps}"

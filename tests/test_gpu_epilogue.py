@@ -103,6 +103,82 @@ def test_bias_dropout_residual_with_dropout(dtype, shape):
     assert torch.equal(rd.grad.cpu(), go)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape,p", [((1024, 1024), 0.2), ((4, 33, 1024), 0.0), ((37, 2560), 0.1),
+                                     ((5, 7, 4096), 0.3), ((19, 8192), 0.1), ((3, 8), 0.5),
+                                     ((130, 1000), 0.1), ((17, 264), 0.0)])
+def test_bias_dropout_residual_layer_norm(dtype, shape, p):
+    """layer_norm(dropout(x + bias) + residual), forward and all five gradients, against the
+    oracle evaluated with torch's own mask (wavefront-per-row and block-per-row kernels, both
+    mask geometries, ragged row counts)."""
+    seed, eps = 2013, 1e-5
+    cols = shape[-1]
+    if dtype == torch.float32 and cols > 4096:
+        pytest.skip("fp32 rows are limited to 4096 columns")
+    x, r, go = _data(shape, dtype)
+    b, w, lb = _data((cols,), dtype, seed=1, n=3)
+    w = (1 + 0.1 * w.float()).to(dtype)
+    keep = None
+    if p > 0:
+        torch.cuda.manual_seed(seed)
+        keep = (F.dropout(torch.ones(shape, device="cuda", dtype=dtype), p) != 0).cpu()
+    xd, bd, rd, wd, lbd = (t.cuda().requires_grad_(True) for t in (x, b, r, w, lb))
+    torch.cuda.manual_seed(seed)
+    out = op.bias_dropout_residual_layer_norm(xd, bd, rd, wd, lbd, p, eps, True)
+    out.backward(go.cuda())
+    # the kernel takes the statistics from z rounded to the tensor type, like the unfused modules
+    y, z, mean, rstd = OE.bias_dropout_residual_layer_norm(x, b, r, w, lb, eps, p, keep,
+                                                           torch.float64, dtype)
+    dx, dbias, dres, dw, dlb = OE.bias_dropout_residual_layer_norm_bwd(go, z, mean, rstd, w, p,
+                                                                       keep, torch.float64)
+    rows = x.numel() // cols
+    assert_parity(out, y, dtype, "y")
+    assert_parity(xd.grad, dx, dtype, "dx")
+    assert_parity(rd.grad, dres, dtype, "dresidual")
+    if p > 0:  # dropped positions carry no gradient, kept ones do (unless dz rounds to zero)
+        assert torch.equal((xd.grad != 0).cpu() & ~keep, torch.zeros_like(keep))
+    for name, got, want in (("dbias", bd.grad, dbias), ("dweight", wd.grad, dw),
+                            ("dln_bias", lbd.grad, dlb)):
+        if dtype == torch.float32:
+            assert max_abs_err(got, want) <= 1e-5 * max(1.0, rows / 16), name
+        else:
+            assert_parity(got, want, dtype, name)
+
+
+def test_layer_norm_fusion_module_and_optional_operands():
+    """The module against nn.LayerNorm on the same parameters; bias / residual left out; no
+    gradient requested (nothing saved); argument errors."""
+    torch.manual_seed(0)
+    ln = torch.nn.LayerNorm(512).cuda()
+    ln.weight.data.normal_(1, 0.1), ln.bias.data.normal_()
+    fused = op.HipBiasDropoutResidualLayerNorm.from_layer_norm(ln, p=0.0)
+    assert fused.weight is ln.weight and fused.bias is ln.bias
+    x, b, r = torch.randn(6, 50, 512, device="cuda"), torch.randn(512, device="cuda"), \
+        torch.randn(6, 50, 512, device="cuda")
+    assert max_abs_err(fused(x, b, r), ln(x + b + r).double()) <= 1e-5
+    assert max_abs_err(fused(x, None, None), ln(x).double()) <= 1e-5
+    assert max_abs_err(fused(x, None, r), ln(x + r).double()) <= 1e-5
+    fused.p = 0.5
+    fused.eval()
+    assert max_abs_err(fused(x, b, r), ln(x + b + r).double()) <= 1e-5
+    fused.train()
+    torch.cuda.manual_seed(3)
+    got = fused(x, b, r)
+    torch.cuda.manual_seed(3)
+    want = ln(F.dropout(x + b, 0.5) + r)
+    assert max_abs_err(got, want.double()) <= 1e-5  # same generator traffic as F.dropout
+    with pytest.raises(ValueError):
+        op.bias_dropout_residual_layer_norm(x, b, r, ln.weight, ln.bias, 1.5)
+    with pytest.raises(ValueError):  # 20000 columns: beyond what a block keeps in registers
+        big = torch.randn(2, 20000, device="cuda")
+        op.bias_dropout_residual_layer_norm(big, None, None, torch.ones(20000, device="cuda"),
+                                            torch.zeros(20000, device="cuda"), 0.0)
+    with pytest.raises(ValueError):  # 1002 columns: not a multiple of the 16-byte vector
+        odd = torch.randn(2, 1002, device="cuda")
+        op.bias_dropout_residual_layer_norm(odd, None, None, torch.ones(1002, device="cuda"),
+                                            torch.zeros(1002, device="cuda"), 0.0)
+
+
 def test_p_one_and_eval_mode():
     x = torch.randn(16, 64, device="cuda")
     b = torch.randn(64, device="cuda")

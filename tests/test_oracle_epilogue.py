@@ -58,3 +58,41 @@ def test_bias_dropout_residual_bwd_is_autograd():
     torch.testing.assert_close(dx, x.grad)
     torch.testing.assert_close(dbias, b.grad)
     torch.testing.assert_close(dres, r.grad)
+
+
+def test_layer_norm_fusion_matches_library_layer_norm_and_autograd():
+    """The written-out LayerNorm against F.layer_norm (library routine) and the closed-form
+    backward against autograd through the library routine; a biased / unbiased variance mix-up,
+    a missing eps or a dropped mean term in dz each fail here."""
+    g = torch.Generator().manual_seed(5)
+    f64 = torch.float64
+    x = torch.randn(4, 9, 12, generator=g, dtype=f64, requires_grad=True)
+    b = torch.randn(12, generator=g, dtype=f64, requires_grad=True)
+    r = torch.randn(4, 9, 12, generator=g, dtype=f64, requires_grad=True)
+    w = torch.randn(12, generator=g, dtype=f64, requires_grad=True)
+    lb = torch.randn(12, generator=g, dtype=f64, requires_grad=True)
+    keep = torch.rand(4, 9, 12, generator=g) > 0.3
+    go = torch.randn(4, 9, 12, generator=g, dtype=f64)
+    eps = 1e-2  # large enough that leaving it out is visible
+    zz = ((x + b) * keep / 0.7 + r)
+    ref = F.layer_norm(zz, (12,), w, lb, eps)
+    ref.backward(go)
+    y, z, mean, rstd = OE.bias_dropout_residual_layer_norm(
+        x.detach(), b.detach(), r.detach(), w.detach(), lb.detach(), eps, 0.3, keep, f64)
+    torch.testing.assert_close(y, ref.detach(), atol=1e-12, rtol=0)
+    torch.testing.assert_close(z, zz.detach())
+    torch.testing.assert_close(mean, zz.detach().mean(-1))
+    torch.testing.assert_close(rstd, 1 / torch.sqrt(zz.detach().var(-1, unbiased=False) + eps))
+    dx, dbias, dres, dw, dlb = OE.bias_dropout_residual_layer_norm_bwd(
+        go, z, mean, rstd, w.detach(), 0.3, keep, f64)
+    for got, want in ((dx, x.grad), (dbias, b.grad), (dres, r.grad), (dw, w.grad), (dlb, lb.grad)):
+        torch.testing.assert_close(got, want, atol=1e-11, rtol=0)
+    # rows that are constant normalise to ln_bias exactly (var = 0, rstd = eps^-1/2)
+    y0 = OE.bias_dropout_residual_layer_norm(torch.full((2, 12), 3.0, dtype=f64), None, None,
+                                             w.detach(), lb.detach(), eps, 0.0, None, f64)[0]
+    torch.testing.assert_close(y0, lb.detach().expand(2, 12))
+    # rounding z first changes the statistics the way a bf16 module's stored sum does
+    yb = OE.bias_dropout_residual_layer_norm(x.detach(), b.detach(), r.detach(), w.detach(),
+                                             lb.detach(), eps, 0.0, None, f64, torch.bfloat16)
+    zb = (x + b + r).detach().to(torch.bfloat16).to(f64)
+    torch.testing.assert_close(yb[0], F.layer_norm(zb, (12,), w.detach(), lb.detach(), eps))
