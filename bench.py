@@ -179,6 +179,42 @@ def bench_epilogues(device, iters=40):
     out["bias_dropout_residual_fwd"] = {"bytes": nbytes, "us": sec * 1e6,
                                         "GBps": nbytes / sec / 1e9,
                                         "frac_of_hbm_peak": nbytes / sec / 1e9 / HBM_PEAK_GBS}
+
+    # bias + dropout + residual + LayerNorm, training form: z, mean, rstd written for the backward
+    zs = [torch.empty(T, Hd, device=device, dtype=bf) for _ in range(n_rot)]
+    gam = torch.ones(Hd, device=device, dtype=bf)
+    bet = torch.zeros(Hd, device=device, dtype=bf)
+    mean = torch.empty(T, device=device, dtype=torch.float32)
+    rstd = torch.empty(T, device=device, dtype=torch.float32)
+
+    def ln_fwd(i):
+        rc = lib.slapo_amd_bias_dropout_residual_ln_fwd(
+            P(xs[i]), P(b1), P(rs[i]), P(gam), P(bet), P(zs[i]), P(os_[i]), P(mean), P(rstd), T,
+            Hd, _lib.SLAPO_BF16, 1e-5, 0.1, 2013, 0, ctypes.byref(plan), st)
+        assert rc == 0
+
+    sec = timed(ln_fwd, n_rot)
+    nbytes = 4 * T * Hd * 2 + 3 * Hd * 2 + 2 * T * 4
+    out["bias_dropout_residual_ln_fwd"] = {"bytes": nbytes, "us": sec * 1e6,
+                                           "GBps": nbytes / sec / 1e9,
+                                           "frac_of_hbm_peak": nbytes / sec / 1e9 / HBM_PEAK_GBS}
+
+    lws_bytes = lib.slapo_amd_ln_bwd_workspace_bytes(T, Hd)
+    lws = torch.empty(lws_bytes // 4, dtype=torch.float32, device=device)
+    dgam, dbet, dbi = (torch.empty(Hd, device=device, dtype=bf) for _ in range(3))
+
+    def ln_bwd(i):  # reads dy (os_), z; writes dx (xs), dresidual (rs) and the three column sums
+        rc = lib.slapo_amd_bias_dropout_residual_ln_bwd(
+            P(os_[i]), P(zs[i]), P(mean), P(rstd), P(gam), P(xs[i]), P(rs[i]), P(dgam), P(dbet),
+            P(dbi), P(lws), lws_bytes, T, Hd, _lib.SLAPO_BF16, 0.1, 2013, 0, ctypes.byref(plan),
+            st)
+        assert rc == 0
+
+    sec = timed(ln_bwd, n_rot)
+    nbytes = 4 * T * Hd * 2 + 4 * Hd * 2 + 2 * T * 4  # partial sums (2 x 6 MB) not credited
+    out["bias_dropout_residual_ln_bwd"] = {"bytes": nbytes, "us": sec * 1e6,
+                                           "GBps": nbytes / sec / 1e9,
+                                           "frac_of_hbm_peak": nbytes / sec / 1e9 / HBM_PEAK_GBS}
     return out
 
 

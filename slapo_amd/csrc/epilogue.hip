@@ -312,7 +312,7 @@ __global__ __launch_bounds__(256) void colsum_finish_kernel(const float* __restr
 // bias + dropout + residual + LayerNorm (the fusion pattern of tests/test_fusion.py:157-204:
 // layer_norm(dropout(x + bias) + residual)).
 //
-// A row is owned by TPR threads: one wavefront (TPR = 64) up to 64 * V * kLnChunks columns, the
+// A row is owned by TPR threads: one wavefront (TPR = 64) up to 64 * V * 2 columns, the
 // whole block (TPR = 256) above, so that every row value stays in registers between the two
 // passes of the statistics and is read from memory once.  z = dropout(x + bias) + residual is
 // rounded to T first and the statistics are taken from the rounded values, i.e. exactly what the
@@ -321,10 +321,27 @@ __global__ __launch_bounds__(256) void colsum_finish_kernel(const float* __restr
 constexpr int kLnChunks = 4;         // 16-byte chunks per thread and row (guarded against cols)
 constexpr int kLnRowsPerBlock = 16;  // backward: rows walked by one block (column partial sums)
 
+// Sum over the 64 lanes, on every lane, without LDS traffic: butterflies inside the 16-lane
+// rows through DPP (quad permutes, row rotations), then the four row sums through v_readlane.
+template <int kCtrl>
+__device__ __forceinline__ float dpp_move(float v) {
+    return __builtin_bit_cast(
+        float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), kCtrl, 0xF, 0xF, false));
+}
 __device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, 64);
-    return v;
+    v += dpp_move<0xB1>(v);   // quad_perm [1,0,3,2]
+    v += dpp_move<0x4E>(v);   // quad_perm [2,3,0,1]
+    v += dpp_move<0x124>(v);  // row_ror 4
+    v += dpp_move<0x128>(v);  // row_ror 8
+    const float r0 = __builtin_bit_cast(
+        float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 0));
+    const float r1 = __builtin_bit_cast(
+        float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 16));
+    const float r2 = __builtin_bit_cast(
+        float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 32));
+    const float r3 = __builtin_bit_cast(
+        float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 48));
+    return (r0 + r1) + (r2 + r3);
 }
 // Sum over the TPR threads of a row.  red: 4 floats of LDS that no other reduction in flight uses
 // (TPR == 256 only; every thread of the block has to call).
@@ -422,45 +439,63 @@ __global__ __launch_bounds__(256) void bias_dropout_residual_ln_fwd_kernel(
 // A block walks kLnRowsPerBlock rows and keeps the three column sums of its threads in
 // registers; they leave as one fp32 partial row triple per block ([block][3][cols]: dgamma, dbeta,
 // dbias) for ln_finish_kernel.  No atomics: the result does not depend on scheduling.
-template <typename T, int V, int TPR, int kDrop>
+// NV = 16-byte chunks per thread and row (1, 2 or 4, the smallest that covers cols): the column
+// sums cost 3 * NV * V registers, and registers decide how many rows a CU has in flight.  The
+// loads of the next two rows are issued before the current row is reduced.
+template <typename T, int V, int NV, int TPR, int kDrop>
 __global__ __launch_bounds__(256) void bias_dropout_residual_ln_bwd_kernel(
     const T* __restrict__ dy, const T* __restrict__ z, const float* __restrict__ mean,
     const float* __restrict__ rstd, const T* __restrict__ gamma, T* __restrict__ dx,
     T* __restrict__ dres, float* __restrict__ partial, int64_t rows, int cols, DropoutState s) {
     constexpr int kRows = 256 / TPR;  // rows in flight per block
     constexpr int kIters = kLnRowsPerBlock / kRows;
-    constexpr int kCombCols = TPR == 64 ? 64 * V * kLnChunks : 1;
+    constexpr int kCombCols = TPR == 64 ? 64 * V * NV : 1;
     __shared__ float red[2][2][4];
-    __shared__ float comb[3 * kCombCols];
+    __shared__ float comb[kRows * 3 * kCombCols];
     const int sub = threadIdx.x % TPR;
     const int rr = threadIdx.x / TPR;
-    Chunk<T, V> gm[kLnChunks];
-    float acc_g[kLnChunks][V], acc_b[kLnChunks][V], acc_x[kLnChunks][V];
+    Chunk<T, V> gm[NV];
+    float acc_g[NV][V], acc_b[NV][V], acc_x[NV][V];
 #pragma unroll
-    for (int u = 0; u < kLnChunks; ++u) {
+    for (int u = 0; u < NV; ++u) {
         const int col0 = (sub + u * TPR) * V;
         if (col0 < cols) gm[u] = load_chunk_cached<T, V>(gamma + col0);
 #pragma unroll
         for (int i = 0; i < V; ++i) acc_g[u][i] = 0.f, acc_b[u][i] = 0.f, acc_x[u][i] = 0.f;
     }
     const float inv_n = 1.0f / (float)cols;
+    const int64_t row0 = (int64_t)blockIdx.x * kLnRowsPerBlock + rr;
+
+    // rows it + 1 and it + 2 are in flight while row it is processed
+    Chunk<T, V> gy[NV], zz[NV], gy_n1[NV], zz_n1[NV], gy_n2[NV], zz_n2[NV];
+    float m = 0.f, rs = 0.f, m_n1 = 0.f, rs_n1 = 0.f, m_n2 = 0.f, rs_n2 = 0.f;
+    auto request = [&](int64_t row, Chunk<T, V> (&g)[NV], Chunk<T, V> (&zc)[NV], float& mm,
+                       float& rr_) __attribute__((always_inline)) {
+        if (row < rows) {  // uniform per wavefront
+            mm = mean[row];
+            rr_ = rstd[row];
+#pragma unroll
+            for (int u = 0; u < NV; ++u) {
+                const int col0 = (sub + u * TPR) * V;
+                if (col0 < cols) {
+                    g[u] = load_chunk<T, V>(dy + row * cols + col0);
+                    zc[u] = load_chunk<T, V>(z + row * cols + col0);
+                }
+            }
+        }
+    };
+    request(row0, gy, zz, m, rs);
+    if (kIters > 1) request(row0 + kRows, gy_n1, zz_n1, m_n1, rs_n1);
 #pragma unroll 1
     for (int it = 0; it < kIters; ++it) {
-        const int64_t row = (int64_t)blockIdx.x * kLnRowsPerBlock + it * kRows + rr;
+        const int64_t row = row0 + it * kRows;
         const bool row_ok = row < rows;  // uniform per wavefront
-        Chunk<T, V> gy[kLnChunks], zz[kLnChunks];
-        float m = 0.f, rs = 0.f, s1 = 0.f, s2 = 0.f;
-        if (row_ok) {
-            m = mean[row];
-            rs = rstd[row];
-        }
+        if (it + 2 < kIters) request(row + 2 * kRows, gy_n2, zz_n2, m_n2, rs_n2);
+        float s1 = 0.f, s2 = 0.f;
 #pragma unroll
-        for (int u = 0; u < kLnChunks; ++u) {
+        for (int u = 0; u < NV; ++u) {
             const int col0 = (sub + u * TPR) * V;
             if (row_ok && col0 < cols) {
-                const int64_t off = row * cols + col0;
-                gy[u] = load_chunk<T, V>(dy + off);
-                zz[u] = load_chunk<T, V>(z + off);
 #pragma unroll
                 for (int i = 0; i < V; ++i) {
                     const float d = Elem<T>::to_f32(gy[u].v[i]);
@@ -476,7 +511,7 @@ __global__ __launch_bounds__(256) void bias_dropout_residual_ln_bwd_kernel(
         const float c1 = row_sum<TPR>(s1, red[it & 1][0]) * inv_n;
         const float c2 = row_sum<TPR>(s2, red[it & 1][1]) * inv_n;
 #pragma unroll
-        for (int u = 0; u < kLnChunks; ++u) {
+        for (int u = 0; u < NV; ++u) {
             const int col0 = (sub + u * TPR) * V;
             if (row_ok && col0 < cols) {
                 const int64_t off = row * cols + col0;
@@ -498,12 +533,18 @@ __global__ __launch_bounds__(256) void bias_dropout_residual_ln_bwd_kernel(
                 if (dx) store_chunk<T, V>(dx + off, ox);
             }
         }
+#pragma unroll
+        for (int u = 0; u < NV; ++u) {
+            gy[u] = gy_n1[u], zz[u] = zz_n1[u];
+            gy_n1[u] = gy_n2[u], zz_n1[u] = zz_n2[u];
+        }
+        m = m_n1, rs = rs_n1, m_n1 = m_n2, rs_n1 = rs_n2;
     }
     if (!partial) return;
     float* out = partial + (int64_t)blockIdx.x * 3 * cols;
     if constexpr (TPR == 256) {
 #pragma unroll
-        for (int u = 0; u < kLnChunks; ++u) {
+        for (int u = 0; u < NV; ++u) {
             const int col0 = (sub + u * TPR) * V;
             if (col0 < cols) {
 #pragma unroll
@@ -515,60 +556,69 @@ __global__ __launch_bounds__(256) void bias_dropout_residual_ln_bwd_kernel(
             }
         }
     } else {
-        // the four wavefronts (row groups) add their sums in turn, then the block writes them
-#pragma unroll 1
-        for (int k = 0; k < kRows; ++k) {
-            if (rr == k) {
+        // every wavefront (row group) parks its sums in LDS, then the block adds the four copies
+        // column by column and writes the partial row with consecutive lanes on consecutive
+        // columns
+        float* mine = comb + rr * 3 * kCombCols;
 #pragma unroll
-                for (int u = 0; u < kLnChunks; ++u) {
-                    const int col0 = (sub + u * TPR) * V;
-                    if (col0 < cols) {
+        for (int u = 0; u < NV; ++u) {
+            const int col0 = (sub + u * TPR) * V;
+            if (col0 < cols) {
 #pragma unroll
-                        for (int i = 0; i < V; ++i) {
-                            const int c = col0 + i;
-                            comb[c] = (k ? comb[c] : 0.f) + acc_g[u][i];
-                            comb[cols + c] = (k ? comb[cols + c] : 0.f) + acc_b[u][i];
-                            comb[2 * cols + c] = (k ? comb[2 * cols + c] : 0.f) + acc_x[u][i];
-                        }
-                    }
+                for (int i = 0; i < V; ++i) {
+                    mine[col0 + i] = acc_g[u][i];
+                    mine[kCombCols + col0 + i] = acc_b[u][i];
+                    mine[2 * kCombCols + col0 + i] = acc_x[u][i];
                 }
             }
-            __syncthreads();
         }
-        for (int c = threadIdx.x; c < 3 * cols; c += 256) out[c] = comb[c];
+        __syncthreads();
+        for (int c = threadIdx.x; c < 3 * cols; c += 256) {
+            const int which = c / cols;
+            const int idx = which * kCombCols + (c - which * cols);
+            out[c] = (comb[idx] + comb[3 * kCombCols + idx]) +
+                     (comb[6 * kCombCols + idx] + comb[9 * kCombCols + idx]);
+        }
     }
 }
 
 // Second stage: partial is [n_partials][3 * cols]; column c of it belongs to dgamma (c < cols),
-// dbeta or dbias.  Same shape of work as colsum_finish_kernel.
-template <typename T>
+// dbeta or dbias.  A block owns kFC columns and kFR row-lanes (kFC * kFR = 256): narrow tiles for
+// small matrices (many blocks, the stage is a chain of L2 round trips), 256-byte segments for
+// large ones (the stage is then bound by reading the partials).
+template <typename T, int kFC, int kFR>
 __global__ __launch_bounds__(256) void ln_finish_kernel(const float* __restrict__ partial,
                                                         T* __restrict__ dgamma,
                                                         T* __restrict__ dbeta,
                                                         T* __restrict__ dbias, int64_t n_partials,
                                                         int cols) {
-    __shared__ float red[kFinRows][kFinCols + 1];
-    const int cx = threadIdx.x % kFinCols;
-    const int ry = threadIdx.x / kFinCols;
+    static_assert(kFC * kFR == 256, "one thread per (column, row-lane)");
+    __shared__ float red[kFR][kFC + 1];
+    const int cx = threadIdx.x % kFC;
+    const int ry = threadIdx.x / kFC;
     const int64_t cols3 = 3 * (int64_t)cols;
-    const int64_t c = (int64_t)blockIdx.x * kFinCols + cx;
+    const int64_t c = (int64_t)blockIdx.x * kFC + cx;
     float t = 0.f;
     if (c < cols3) {
-        float t0 = 0.f, t1 = 0.f;
+        // eight loads in flight per thread
+        float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         int64_t k = ry;
-        for (; k + kFinRows < n_partials; k += 2 * kFinRows) {
-            t0 += partial[k * cols3 + c];
-            t1 += partial[(k + kFinRows) * cols3 + c];
+        for (; k + 7 * kFR < n_partials; k += 8 * kFR) {
+            float v[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = partial[(k + j * kFR) * cols3 + c];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) acc[j] += v[j];
         }
-        for (; k < n_partials; k += kFinRows) t0 += partial[k * cols3 + c];
-        t = t0 + t1;
+        for (; k < n_partials; k += kFR) acc[0] += partial[k * cols3 + c];
+        t = ((acc[0] + acc[1]) + (acc[2] + acc[3])) + ((acc[4] + acc[5]) + (acc[6] + acc[7]));
     }
     red[ry][cx] = t;
     __syncthreads();
     if (ry == 0 && c < cols3) {
         float sum = 0.f;
 #pragma unroll
-        for (int r = 0; r < kFinRows; ++r) sum += red[r][cx];
+        for (int r = 0; r < kFR; ++r) sum += red[r][cx];
         const int which = (int)(c / cols);
         T* dst = which == 0 ? dgamma : which == 1 ? dbeta : dbias;
         if (dst) dst[c - (int64_t)which * cols] = Elem<T>::from_f32(sum);
@@ -741,7 +791,7 @@ inline int ln_geometry(int64_t rows, int64_t cols, bool* wide) {
     constexpr int V = Elem<T>::kPerVec;
     if (cols % V != 0) return SLAPO_ERR_ALIGN;
     if (cols > 256 * V * kLnChunks) return SLAPO_ERR_SHAPE;
-    *wide = cols > 64 * V * kLnChunks;
+    *wide = cols > 64 * V * 2;  // a wavefront per row up to two chunks per lane, a block above
     if (rows > 0x7FFFFFFF) return SLAPO_ERR_SHAPE;
     return SLAPO_OK;
 }
@@ -791,26 +841,45 @@ int ln_bwd_dispatch(const void* dy, const void* z, const float* mean, const floa
     const int64_t n_blocks = (rows + kLnRowsPerBlock - 1) / kLnRowsPerBlock;
     float* partial = want_sums ? (float*)ws : nullptr;
     const int mode = !dropout ? 0 : (s.g_shift >= 0 && s.t_shift >= 0) ? 1 : 2;
-#define SLAPO_LAUNCH_LNB(TPR, MODE)                                                             \
-    hipLaunchKernelGGL((bias_dropout_residual_ln_bwd_kernel<T, V, TPR, MODE>),                  \
+#define SLAPO_LAUNCH_LNB(NV, TPR, MODE)                                                         \
+    hipLaunchKernelGGL((bias_dropout_residual_ln_bwd_kernel<T, V, NV, TPR, MODE>),              \
                        dim3((unsigned)n_blocks), dim3(256), 0, st, (const T*)dy, (const T*)z,   \
                        mean, rstd, (const T*)gamma, (T*)dx, (T*)dres, partial, rows, (int)cols, \
                        s)
+#define SLAPO_LAUNCH_LNB_MODE(NV, TPR)            \
+    do {                                          \
+        if (mode == 0) SLAPO_LAUNCH_LNB(NV, TPR, 0); \
+        if (mode == 1) SLAPO_LAUNCH_LNB(NV, TPR, 1); \
+        if (mode == 2) SLAPO_LAUNCH_LNB(NV, TPR, 2); \
+    } while (0)
+    const int tpr = wide ? 256 : 64;
+    const int chunks = (int)((cols / V + tpr - 1) / tpr);  // per thread and row, 1..kLnChunks
     if (wide) {
-        if (mode == 0) SLAPO_LAUNCH_LNB(256, 0);
-        if (mode == 1) SLAPO_LAUNCH_LNB(256, 1);
-        if (mode == 2) SLAPO_LAUNCH_LNB(256, 2);
+        if (chunks <= 1)
+            SLAPO_LAUNCH_LNB_MODE(1, 256);
+        else if (chunks <= 2)
+            SLAPO_LAUNCH_LNB_MODE(2, 256);
+        else
+            SLAPO_LAUNCH_LNB_MODE(4, 256);
     } else {
-        if (mode == 0) SLAPO_LAUNCH_LNB(64, 0);
-        if (mode == 1) SLAPO_LAUNCH_LNB(64, 1);
-        if (mode == 2) SLAPO_LAUNCH_LNB(64, 2);
+        if (chunks <= 1)
+            SLAPO_LAUNCH_LNB_MODE(1, 64);
+        else
+            SLAPO_LAUNCH_LNB_MODE(2, 64);
     }
+#undef SLAPO_LAUNCH_LNB_MODE
 #undef SLAPO_LAUNCH_LNB
     rc = check_launch();
     if (rc != SLAPO_OK || !want_sums) return rc;
-    const unsigned blocks = (unsigned)((3 * cols + kFinCols - 1) / kFinCols);
-    hipLaunchKernelGGL((ln_finish_kernel<T>), dim3(blocks), dim3(256), 0, st, partial,
-                       (T*)dgamma, (T*)dbeta, (T*)dbias, n_blocks, (int)cols);
+    if (3 * cols >= 6144) {
+        hipLaunchKernelGGL((ln_finish_kernel<T, 64, 4>), dim3((unsigned)((3 * cols + 63) / 64)),
+                           dim3(256), 0, st, partial, (T*)dgamma, (T*)dbeta, (T*)dbias, n_blocks,
+                           (int)cols);
+    } else {
+        hipLaunchKernelGGL((ln_finish_kernel<T, 16, 16>), dim3((unsigned)((3 * cols + 15) / 16)),
+                           dim3(256), 0, st, partial, (T*)dgamma, (T*)dbeta, (T*)dbias, n_blocks,
+                           (int)cols);
+    }
     return check_launch();
 }
 
