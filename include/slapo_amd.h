@@ -160,6 +160,28 @@ int slapo_amd_bias_dropout_residual_ln_bwd(const void* grad_y, const void* z, co
                                            const slapo_dropout_plan* plan, void* stream);
 
 /* ------------------------------------------------------------------------------------------
+ * Vocab-parallel cross entropy, the part computed on one shard [rows, vocab] of the logits
+ * (vocabulary ids vocab_start .. vocab_start + vocab - 1).  Replaces the tensor passes of
+ * _VocabParallelCrossEntropy.forward / .backward (slapo/op/cross_entropy.py:21-124).
+ *
+ * Forward, one read of the logits: per row the local maximum row_max, sum_exp = sum exp(x -
+ * row_max), predicted = logit of target[row] if it lies in this shard (else 0) and sum_logits =
+ * sum x (for label smoothing); all fp32 [rows].  The tensor-parallel group combines them as
+ * M = max row_max, S = sum sum_exp * exp(row_max - M), P = sum predicted (the reference's three
+ * all-reduces, :25, :56, :62), loss = log S + M - P.
+ * Backward, one read and one write: grad_logits = grad_loss * (exp(x - row_max) * inv_sum_exp
+ * - [v == target] * (1 - s) - s / vocab) with the COMBINED row_max = M and inv_sum_exp = 1 / S and
+ * s = label_smoothing * vocab / (vocab - 1) (:112-122).  target is int64; any dtype of SLAPO_*;
+ * rows need no alignment beyond that of an element. */
+int slapo_amd_vocab_ce_fwd(const void* logits, const int64_t* target, float* row_max,
+                           float* sum_exp, float* predicted, float* sum_logits, int64_t rows,
+                           int64_t vocab, int64_t vocab_start, int dtype, void* stream);
+int slapo_amd_vocab_ce_bwd(const void* logits, const int64_t* target, const float* row_max,
+                           const float* inv_sum_exp, const float* grad_loss, void* grad_logits,
+                           int64_t rows, int64_t vocab, int64_t vocab_start,
+                           double label_smoothing, int dtype, void* stream);
+
+/* ------------------------------------------------------------------------------------------
  * Attention:  O = dropout(softmax(Q K^T * scale + bias + mask)) V, forward and backward.
  *
  * Replaces: the attn_fn callees of FlashAttentionOp.forward -- xformers

@@ -112,6 +112,15 @@ PROTOTYPES = {
          c_i64, c_i64, ctypes.c_int, ctypes.c_double, c_u64, c_u64,
          ctypes.POINTER(DropoutPlan), c_vp],
     ),
+    "slapo_amd_vocab_ce_fwd": (
+        ctypes.c_int,
+        [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, ctypes.c_int, c_vp],
+    ),
+    "slapo_amd_vocab_ce_bwd": (
+        ctypes.c_int,
+        [c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_i64, c_i64, c_i64, ctypes.c_double, ctypes.c_int,
+         c_vp],
+    ),
     "slapo_amd_attn_fwd": (
         ctypes.c_int, [ctypes.POINTER(AttnParams), c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp]
     ),

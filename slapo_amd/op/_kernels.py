@@ -203,6 +203,44 @@ def bias_dropout_residual_ln_bwd(grad, z, mean, rstd, weight, p, seed, offset, p
     return outs
 
 
+def vocab_ce_fwd(logits, target, vocab_start=0):
+    """Per-row (row_max, sum_exp, predicted, sum_logits) of one vocabulary shard, fp32 [rows]."""
+    _require_device(logits, target)
+    logits = logits.contiguous()
+    vocab = logits.shape[-1]
+    rows = logits.numel() // max(vocab, 1)
+    target = target.contiguous().view(-1).to(torch.int64)
+    if target.numel() != rows:
+        raise ValueError("target must have the shape of the logits without the vocabulary dim")
+    stats = torch.empty(4, max(rows, 1), dtype=torch.float32, device=logits.device)
+    if rows:
+        with torch.cuda.device(logits.device):
+            rc = _lib.load().slapo_amd_vocab_ce_fwd(
+                _ptr(logits), _ptr(target), _ptr(stats[0]), _ptr(stats[1]), _ptr(stats[2]),
+                _ptr(stats[3]), rows, vocab, int(vocab_start), _lib.dtype_code(logits.dtype),
+                _stream())
+        _lib.check(rc, "slapo_amd_vocab_ce_fwd")
+    return stats[0, :rows], stats[1, :rows], stats[2, :rows], stats[3, :rows], logits, target
+
+
+def vocab_ce_bwd(logits, target, row_max, inv_sum_exp, grad_loss, vocab_start=0,
+                 label_smoothing=0.0):
+    _require_device(logits, target, row_max, inv_sum_exp, grad_loss)
+    vocab = logits.shape[-1]
+    rows = logits.numel() // max(vocab, 1)
+    grad = torch.empty_like(logits)
+    grad_loss = grad_loss.contiguous().view(-1).float()
+    if rows:
+        with torch.cuda.device(logits.device):
+            rc = _lib.load().slapo_amd_vocab_ce_bwd(
+                _ptr(logits), _ptr(target), _ptr(row_max.contiguous()),
+                _ptr(inv_sum_exp.contiguous()), _ptr(grad_loss), _ptr(grad), rows, vocab,
+                int(vocab_start), float(label_smoothing), _lib.dtype_code(logits.dtype),
+                _stream())
+        _lib.check(rc, "slapo_amd_vocab_ce_bwd")
+    return grad
+
+
 def dropout_mask(numel, elem_bytes, p, seed, offset, device):
     """Boolean keep-mask [numel] drawn on the device (debugging / test aid)."""
     plan = dropout_plan(numel, elem_bytes, device)
