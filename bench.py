@@ -215,6 +215,36 @@ def bench_epilogues(device, iters=40):
     out["bias_dropout_residual_ln_bwd"] = {"bytes": nbytes, "us": sec * 1e6,
                                            "GBps": nbytes / sec / 1e9,
                                            "frac_of_hbm_peak": nbytes / sec / 1e9 / HBM_PEAK_GBS}
+    del xs, rs, os_, zs
+
+    # vocab-parallel cross entropy on one shard: GPT-2's unpadded vocabulary, fp16 logits
+    V = 50257
+    logits = torch.randn(T, V, device=device, dtype=torch.float16)
+    grad = torch.empty_like(logits)
+    tgt = torch.randint(0, V, (T,), device=device)
+    stats = torch.empty(4, T, device=device, dtype=torch.float32)
+    gl = torch.ones(T, device=device, dtype=torch.float32)
+
+    def ce_fwd(i):
+        rc = lib.slapo_amd_vocab_ce_fwd(P(logits), P(tgt), P(stats[0]), P(stats[1]), P(stats[2]),
+                                        P(stats[3]), T, V, 0, _lib.SLAPO_F16, st)
+        assert rc == 0
+
+    sec = timed(ce_fwd, 1)
+    nbytes = T * V * 2 + T * (8 + 16)
+    out["vocab_ce_fwd"] = {"bytes": nbytes, "us": sec * 1e6, "GBps": nbytes / sec / 1e9,
+                           "frac_of_hbm_peak": nbytes / sec / 1e9 / HBM_PEAK_GBS}
+    inv_s = 1.0 / stats[1]
+
+    def ce_bwd(i):
+        rc = lib.slapo_amd_vocab_ce_bwd(P(logits), P(tgt), P(stats[0]), P(inv_s), P(gl), P(grad),
+                                        T, V, 0, 0.0, _lib.SLAPO_F16, st)
+        assert rc == 0
+
+    sec = timed(ce_bwd, 1)
+    nbytes = 2 * T * V * 2 + T * (8 + 12)
+    out["vocab_ce_bwd"] = {"bytes": nbytes, "us": sec * 1e6, "GBps": nbytes / sec / 1e9,
+                           "frac_of_hbm_peak": nbytes / sec / 1e9 / HBM_PEAK_GBS}
     return out
 
 

@@ -1,7 +1,8 @@
 """CPU oracle for the Slapo fused-op hot path.  TEST INFRASTRUCTURE ONLY.
 
 This package restates, on the CPU, the arithmetic of the reference's native PyTorch path
-(awslabs/slapo, slapo/op/attention.py and slapo/op/fused_bias.py) and of the Philox dropout
+(awslabs/slapo, slapo/op/attention.py, slapo/op/fused_bias.py, slapo/op/cross_entropy.py and
+the LayerNorm fusion pattern of tests/test_fusion.py:157-204) and of the Philox dropout
 mask that torch.nn.functional.dropout draws on a ROCm device.  Only tests/, the smoke check in
 __graft_entry__.py and the cpu_baseline leg of bench.py may import it; the product package
 (slapo_amd) never does and has no CPU path of its own.
@@ -21,6 +22,13 @@ What pins each function (none of them is pinned by retyping its own formula):
   epilogue.bias_dropout(_residual)
       identity at p = 0; at p > 0 the explicit-mask semantics of flash_attn_ref
       (masked_fill(~mask, 0) and scaling by 1/(1-p), slapo/op/attention.py:118-125).
+  epilogue.bias_dropout_residual_layer_norm(_bwd)
+      torch.nn.functional.layer_norm (library routine) and autograd through it, with an eps large
+      enough that leaving it out shows; constant rows (exactly ln_bias).
+  cross_entropy.forward / backward / shard_stats / combine
+      torch.nn.functional.cross_entropy (library routine; its label smoothing equals the
+      reference's at alpha K / (K - 1)), autograd, and the identity between the whole-vocabulary
+      loss and the loss combined from shard statistics for several cuts.
   philox.philox4x32_10
       the Random123 known-answer vectors for Philox4x32-10.
   philox.aten_dropout_mask (element -> subsequence/counter/lane mapping)
