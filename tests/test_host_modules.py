@@ -112,6 +112,42 @@ def test_no_cpu_fallback():
     mlp = op.FusedMLP(8, 32, "gelu", 0.0)
     with pytest.raises(RuntimeError, match="gfx950"):
         mlp(torch.zeros(2, 8))
+    with pytest.raises(RuntimeError, match="gfx950"):
+        op.bias_dropout_residual_layer_norm(torch.zeros(4, 8), torch.zeros(8), torch.zeros(4, 8),
+                                            torch.ones(8), torch.zeros(8), 0.0)
+    with pytest.raises(RuntimeError, match="gfx950"):
+        op.ParallelCrossEntropy()(torch.zeros(4, 8), torch.zeros(4, dtype=torch.long))
+
+
+def test_layer_norm_fusion_module_and_cross_entropy_interfaces():
+    """The LayerNorm payload carries nn.LayerNorm's parameter names (a state_dict of the module it
+    replaces loads into it); ParallelCrossEntropy keeps the reference's constructor and forward
+    (slapo/op/cross_entropy.py:153-160) and its helper for the vocabulary range (:11-14)."""
+    ln = nn.LayerNorm(16, eps=1e-6)
+    fused = op.HipBiasDropoutResidualLayerNorm.from_layer_norm(ln, p=0.25)
+    assert fused.weight is ln.weight and fused.bias is ln.bias
+    assert (fused.p, fused.eps, fused.normalized_shape) == (0.25, 1e-6, (16,))
+    fresh = op.HipBiasDropoutResidualLayerNorm(16, 0.1)
+    fresh.load_state_dict(ln.state_dict())
+    assert _params(fresh.forward) == [("x", inspect.Parameter.empty),
+                                      ("bias", inspect.Parameter.empty),
+                                      ("residual", inspect.Parameter.empty)]
+    with pytest.raises(ValueError):
+        op.HipBiasDropoutResidualLayerNorm(16, 1.5)
+    with pytest.raises(NotImplementedError):
+        op.HipBiasDropoutResidualLayerNorm((4, 16), 0.1)
+    with pytest.raises(NotImplementedError):
+        op.HipBiasDropoutResidualLayerNorm.from_layer_norm(
+            nn.LayerNorm(16, elementwise_affine=False), 0.1)
+
+    from slapo_amd.op import cross_entropy as CE
+
+    assert _params(op.ParallelCrossEntropy.__init__) == [("group", None)]
+    assert [n for n, _ in _params(op.ParallelCrossEntropy.forward)] == ["outputs", "labels"]
+    assert _params(op.vocab_parallel_cross_entropy) == [
+        ("vocab_parallel_logits", inspect.Parameter.empty), ("target", inspect.Parameter.empty),
+        ("label_smoothing", 0.0), ("group", None)]
+    assert CE.vocab_range_from_per_partition_vocab_size(100, 3, 8) == (300, 400)
 
 
 def test_meta_device_construction():
