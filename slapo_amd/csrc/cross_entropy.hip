@@ -76,7 +76,7 @@ __global__ __launch_bounds__(kCeThreads) void ce_fwd_kernel(
     if ((int)threadIdx.x < sp.head) add1(Elem<T>::to_f32(x[threadIdx.x]));
     for (int e = sp.tail0 + threadIdx.x; e < n; e += kCeThreads) add1(Elem<T>::to_f32(x[e]));
     const T* body = x + sp.head;
-    for (int i = threadIdx.x; i < sp.nvec; i += kCeThreads) {
+    auto load_vec = [&](int i) __attribute__((always_inline)) -> CeVec<T, V> {
         CeVec<T, V> c;
         if constexpr (V == 1) {
             c.v[0] = body[i];
@@ -84,6 +84,9 @@ __global__ __launch_bounds__(kCeThreads) void ce_fwd_kernel(
             *reinterpret_cast<u32x4_t*>(&c) =
                 __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(body) + i);
         }
+        return c;
+    };
+    auto take_vec = [&](const CeVec<T, V>& c) __attribute__((always_inline)) {
         float f[V];
         float vm = -INFINITY;
 #pragma unroll
@@ -103,7 +106,17 @@ __global__ __launch_bounds__(kCeThreads) void ce_fwd_kernel(
             for (int j = 0; j < V; ++j)
                 s += __builtin_amdgcn_exp2f((f[j] - m) * 1.4426950408889634f);
         }
+    };
+    // four loads in flight per thread
+    int i = threadIdx.x;
+    for (; i + 3 * kCeThreads < sp.nvec; i += 4 * kCeThreads) {
+        CeVec<T, V> c[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) c[u] = load_vec(i + u * kCeThreads);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) take_vec(c[u]);
     }
+    for (; i < sp.nvec; i += kCeThreads) take_vec(load_vec(i));
     // block reduction: butterflies inside the wavefront, then the four wavefronts through LDS
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) {
@@ -148,41 +161,58 @@ __global__ __launch_bounds__(kCeThreads) void ce_bwd_kernel(
     T* dx = grad + row * (int64_t)n;
     const RowSplit<T> sp = split_row<T, V>(x, n);
     const float mx = row_max[row];
-    const float is = inv_sum[row];
     const float g = grad_loss[row];
-    const int64_t t64 = target[row] - vocab_start;
-    const int t = (t64 >= 0 && t64 < n) ? (int)t64 : -1;
-    auto one = [&](float v, int e) __attribute__((always_inline)) -> float {
-        // v - max first: exact for logits near the maximum even when both sit far from zero
-        float p = __builtin_amdgcn_exp2f((v - mx) * 1.4426950408889634f) * is - flat;
-        if (e == t) p -= onehot_scale;
-        return p * g;
+    const float isg = inv_sum[row] * g;
+    const float flatg = flat * g;
+    // (softmax - flat) g; the target's element is corrected after the stream, so that the loop
+    // carries no comparison.  v - max first: exact for logits near the maximum even when both
+    // sit far from zero.
+    auto one = [&](float v) __attribute__((always_inline)) -> float {
+        return __builtin_fmaf(__builtin_amdgcn_exp2f((v - mx) * 1.4426950408889634f), isg, -flatg);
     };
     if ((int)threadIdx.x < sp.head)
-        dx[threadIdx.x] = Elem<T>::from_f32(one(Elem<T>::to_f32(x[threadIdx.x]), threadIdx.x));
+        dx[threadIdx.x] = Elem<T>::from_f32(one(Elem<T>::to_f32(x[threadIdx.x])));
     for (int e = sp.tail0 + threadIdx.x; e < n; e += kCeThreads)
-        dx[e] = Elem<T>::from_f32(one(Elem<T>::to_f32(x[e]), e));
+        dx[e] = Elem<T>::from_f32(one(Elem<T>::to_f32(x[e])));
     const T* body = x + sp.head;
     T* obody = dx + sp.head;
-    for (int i = threadIdx.x; i < sp.nvec; i += kCeThreads) {
-        CeVec<T, V> c, o;
+    auto load_vec = [&](int i) __attribute__((always_inline)) -> CeVec<T, V> {
+        CeVec<T, V> c;
         if constexpr (V == 1) {
             c.v[0] = body[i];
         } else {
             *reinterpret_cast<u32x4_t*>(&c) =
                 __builtin_nontemporal_load(reinterpret_cast<const u32x4_t*>(body) + i);
         }
-        const int e0 = sp.head + i * V;
+        return c;
+    };
+    auto emit_vec = [&](int i, const CeVec<T, V>& c) __attribute__((always_inline)) {
+        CeVec<T, V> o;
 #pragma unroll
-        for (int j = 0; j < V; ++j)
-            o.v[j] = Elem<T>::from_f32(one(Elem<T>::to_f32(c.v[j]), e0 + j));
+        for (int j = 0; j < V; ++j) o.v[j] = Elem<T>::from_f32(one(Elem<T>::to_f32(c.v[j])));
         if constexpr (V == 1) {
             obody[i] = o.v[0];
         } else {
             __builtin_nontemporal_store(*reinterpret_cast<const u32x4_t*>(&o),
                                         reinterpret_cast<u32x4_t*>(obody) + i);
         }
+    };
+    // four loads in flight per thread
+    int i = threadIdx.x;
+    for (; i + 3 * kCeThreads < sp.nvec; i += 4 * kCeThreads) {
+        CeVec<T, V> c[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) c[u] = load_vec(i + u * kCeThreads);
+#pragma unroll
+        for (int u = 0; u < 4; ++u) emit_vec(i + u * kCeThreads, c[u]);
     }
+    for (; i < sp.nvec; i += kCeThreads) emit_vec(i, load_vec(i));
+    // the one-hot term of the target, if it lies in this shard: written after every thread of
+    // the block has stored its part of the row
+    const int64_t t64 = target[row] - vocab_start;
+    __syncthreads();
+    if (threadIdx.x == 0 && t64 >= 0 && t64 < n)
+        dx[t64] = Elem<T>::from_f32(one(Elem<T>::to_f32(x[t64])) - onehot_scale * g);
 }
 
 inline bool ce_dims_ok(int64_t rows, int64_t n) {
