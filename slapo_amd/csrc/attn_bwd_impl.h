@@ -165,18 +165,43 @@ __global__ __launch_bounds__(kBwdThreads, ((DPAD <= 64 && KB == 1) ? 2 : 1)) voi
     const int a_off = pi_row(c_loc) * kPitch + 8 * g;
     const int t_off = (8 * g + ((lane & 15) >> 2)) * kPitch + ((lane >> 4) & 1) * 16 + 4 * (lane & 3);
 
-    QStage qst, gst;
-    qst.init(a.qs[1], a.d);
-    gst.init(a.os[1], a.d);
-    // lse / delta of a query tile: threads 0..63 fetch lse, threads 64..127 delta.  The load is
-    // unconditional (row clamped) and its result is not touched until the tile is written to LDS.
-    float stat_reg = 0.f;
-    const float* stat_src = (threadIdx.x < kBwdBM) ? lse_base : delta_base;
-    auto load_stats = [&](int i0) __attribute__((always_inline)) {
-        if (threadIdx.x < 2 * kBwdBM)
-            stat_reg = stat_src[min(i0 + (int)(threadIdx.x & (kBwdBM - 1)), a.sq - 1)];
+    // Registers through which a query tile (Q, dO rows, lse / delta, keep bits) travels from
+    // global memory to LDS.
+    struct TileRegs {
+        QStage q, g;
+        float stat;
+        uint32_t mask;
     };
-    auto store_stats = [&](int buf, int i0) __attribute__((always_inline)) {
+    TileRegs regs;
+    regs.q.init(a.qs[1], a.d);
+    regs.g.init(a.os[1], a.d);
+    regs.stat = 0.f, regs.mask = 0u;
+    // lse / delta of a query tile: threads 0..63 fetch lse, threads 64..127 delta.
+    const float* stat_src = (threadIdx.x < kBwdBM) ? lse_base : delta_base;
+    // Requests tile t.  Unconditional: rows are clamped into the tensor (past the last tile the
+    // request is wasted), so it stays straight-line code; nothing is touched until stage_tile.
+    auto request_tile = [&](TileRegs& r, int t) __attribute__((always_inline)) {
+        const int i0 = t * kBwdBM;
+        r.q.load(q_base, a.qs[1], i0, a.sq, a.d);
+        r.g.load(g_base, a.os[1], i0, a.sq, a.d);
+        if (threadIdx.x < 2 * kBwdBM)
+            r.stat = stat_src[min(i0 + (int)(threadIdx.x & (kBwdBM - 1)), a.sq - 1)];
+        if constexpr (kDrop == 3) {
+            // the keep bits that the forward stored: thread (w, row) of the workgroup fetches the
+            // word of query row i0 + row for the 32 keys of wavefront w
+            const int w = min((k0 >> 5) + (int)(threadIdx.x >> 6), a.mask_words - 1);
+            const int row = min(i0 + (int)(threadIdx.x & 63), a.mask_pitch - 1);
+            r.mask = a.keep_mask[((int64_t)bh * a.mask_words + w) * a.mask_pitch + row];
+        }
+    };
+    // Writes the requested tile t into its LDS buffer (tiles alternate between two buffers).
+    auto stage_tile = [&](TileRegs& r, int t) __attribute__((always_inline)) {
+        const int buf = (t - t_lo) & 1;
+        const int i0 = t * kBwdBM;
+        r.q.fix(i0, a.sq, a.d);
+        r.g.fix(i0, a.sq, a.d);
+        r.q.store(q_lds + buf * SM::kQTile);
+        r.g.store(g_lds + buf * SM::kQTile);
         if (threadIdx.x < 2 * kBwdBM) {
             const bool ok = i0 + (int)(threadIdx.x & (kBwdBM - 1)) < a.sq;
             // lse in units of the raw dot product (lse / scale), so that exp2(scale_log2 * (s - lse))
@@ -187,35 +212,31 @@ __global__ __launch_bounds__(kBwdThreads, ((DPAD <= 64 && KB == 1) ? 2 : 1)) voi
             float v;
             if constexpr (kFold)
                 v = (threadIdx.x < kBwdBM)
-                        ? (ok ? fmaxf(fminf(stat_reg * inv_scale, kNoRow), -kNoRow) : kNoRow)
-                        : (ok ? stat_reg : 0.f);
+                        ? (ok ? fmaxf(fminf(r.stat * inv_scale, kNoRow), -kNoRow) : kNoRow)
+                        : (ok ? r.stat : 0.f);
             else  // lse in log2 units, +inf past the end
-                v = (threadIdx.x < kBwdBM) ? (ok ? stat_reg * kLog2e : INFINITY)
-                                           : (ok ? stat_reg : 0.f);
+                v = (threadIdx.x < kBwdBM) ? (ok ? r.stat * kLog2e : INFINITY)
+                                           : (ok ? r.stat : 0.f);
             stat_lds[buf * 2 * kBwdBM + threadIdx.x] = v;
         }
+        if constexpr (kDrop == 3) mask_lds[buf * kBwdThreads + threadIdx.x] = r.mask;
     };
+    auto tile_fast = [&](int t) __attribute__((always_inline)) {
+        const int i0 = t * kBwdBM;
+        return a.window <= 0 && k0 + kBN <= a.sk && i0 + kBwdBM <= a.sq &&
+               (!a.causal || i0 >= k0 + kBN - 1);
+    };
+    // Two generic (diagonal / tail) tiles in a row are processed together, see generic_step; when
+    // the kernel starts with such a pair, both tiles are requested at once.
+    // (Measured: 3.5 % on the kernel at head_dim 128, 15 % with a local window; at 64 the second
+    // register set spills and costs more than the pairing saves, at 80 it is a wash.)
+    constexpr bool kPairGeneric = DPAD > 96;
+    const bool pair_first =
+        kPairGeneric && t_lo + 1 < t_hi && !tile_fast(t_lo) && !tile_fast(t_lo + 1);
+    TileRegs second = regs;  // same lane offsets
 
-    // kDrop == 3: the keep bits that the forward stored.  Thread (w, row) of the workgroup fetches
-    // the word of query row i0 + row for the 32 keys of wavefront w; the tile goes through LDS
-    // like lse / delta.
-    uint32_t mask_reg = 0u;
-    auto load_mask = [&](int i0) __attribute__((always_inline)) {
-        if constexpr (kDrop == 3) {
-            const int w = min((k0 >> 5) + (int)(threadIdx.x >> 6), a.mask_words - 1);
-            const int row = min(i0 + (int)(threadIdx.x & 63), a.mask_pitch - 1);
-            mask_reg = a.keep_mask[((int64_t)bh * a.mask_words + w) * a.mask_pitch + row];
-        }
-    };
-    auto store_mask = [&](int buf) __attribute__((always_inline)) {
-        if constexpr (kDrop == 3) mask_lds[buf * kBwdThreads + threadIdx.x] = mask_reg;
-    };
-
-    // rows are clamped into the tensor, so the request is safe even without any query tile
-    qst.load(q_base, a.qs[1], t_lo * kBwdBM, a.sq, a.d);
-    gst.load(g_base, a.os[1], t_lo * kBwdBM, a.sq, a.d);
-    load_stats(t_lo * kBwdBM);
-    load_mask(t_lo * kBwdBM);
+    request_tile(regs, t_lo);
+    if constexpr (kPairGeneric) request_tile(second, t_lo + 1);
 #pragma unroll
     for (int kb = 0; kb < KB; ++kb)
 #pragma unroll
@@ -224,13 +245,9 @@ __global__ __launch_bounds__(kBwdThreads, ((DPAD <= 64 && KB == 1) ? 2 : 1)) voi
             kf[kb][t] = __builtin_bit_cast(frag_t, keep_or_zero(k_raw[kb][t], keep));
             vf[kb][t] = __builtin_bit_cast(frag_t, keep_or_zero(v_raw[kb][t], keep));
         }
-    if (t_lo < t_hi) {
-        qst.fix(t_lo * kBwdBM, a.sq, a.d);
-        gst.fix(t_lo * kBwdBM, a.sq, a.d);
-        qst.store(q_lds);
-        gst.store(g_lds);
-        store_stats(0, t_lo * kBwdBM);
-        store_mask(0);
+    if (t_lo < t_hi) stage_tile(regs, t_lo);
+    if constexpr (kPairGeneric) {
+        if (pair_first) stage_tile(second, t_lo + 1);
     }
     __syncthreads();
 
@@ -446,11 +463,9 @@ __global__ __launch_bounds__(kBwdThreads, ((DPAD <= 64 && KB == 1) ? 2 : 1)) voi
         }
     };
 
-    // Iteration t: request tile t+1, process tile t, write tile t+1 into the other buffer.
-    // kFast iterations hold tiles in which every key of the workgroup sees every query, so their
-    // body is one straight block; the others test activity and masks per wavefront and half.
-    auto iteration = [&](int t, auto fast_tag) __attribute__((always_inline)) {
-        constexpr bool kFast = decltype(fast_tag)::value;
+    // Fast iteration t (every key of the workgroup sees every query of the tile): request tile
+    // t+1, process tile t as one straight block, write tile t+1 into the other buffer.
+    auto fast_iteration = [&](int t) __attribute__((always_inline)) {
         const int buf = (t - t_lo) & 1;
         const T* qt = q_lds + buf * SM::kQTile;
         const T* gt = g_lds + buf * SM::kQTile;
@@ -458,77 +473,89 @@ __global__ __launch_bounds__(kBwdThreads, ((DPAD <= 64 && KB == 1) ? 2 : 1)) voi
         const float* delta_t = lse_t + kBwdBM;
         const uint32_t* mask_t = mask_lds + buf * kBwdThreads + wave * kBwdBM;
         const int i0 = t * kBwdBM;
-        const bool have_next = t + 1 < t_hi;
-        // The next tile is requested unconditionally (rows are clamped into the tensor; after the
-        // last tile the request is wasted) so that the request stays straight-line code.  In the
-        // fast body it is issued in the middle, once the score registers of the first half are
-        // dead, which keeps the staging registers out of the busiest stretch.
-        auto request_next = [&]() __attribute__((always_inline)) {
-            qst.load(q_base, a.qs[1], i0 + kBwdBM, a.sq, a.d);
-            gst.load(g_base, a.os[1], i0 + kBwdBM, a.sq, a.d);
-            load_stats(i0 + kBwdBM);
-            load_mask(i0 + kBwdBM);
-        };
-        // (only where two workgroups share a CU and registers are the scarce resource)
-        constexpr bool kLateRequest = kFast && DPAD <= 64;
-        if constexpr (!kLateRequest) request_next();
-        if constexpr (kFast) {
-            std::integral_constant<int, 0> none;
-            f32x16_t s0[KB], s1[KB], p0[KB], p1[KB];
-            uint32_t pw0[KB][8], dw0[KB][8], pw1[KB][8], dw1[KB][8];
-            half_sp(qt, gt, lse_t, delta_t, 0, s0, p0);
-            half_exp(s0, lse_t, i0, none);
-            half_sp(qt, gt, lse_t + 32, delta_t + 32, 1, s1, p1);
-            half_ds(s0, p0, delta_t, mask_t, i0, pw0, dw0);
-            half_exp(s1, lse_t + 32, i0 + 32, none);
-            if constexpr (kLateRequest) {
-                __builtin_amdgcn_sched_barrier(0);
-                request_next();
-                __builtin_amdgcn_sched_barrier(0);
-            }
-            half_out(qt, gt, 0, pw0, dw0);
-            half_ds(s1, p1, delta_t + 32, mask_t + 32, i0 + 32, pw1, dw1);
-            half_out(qt, gt, 1, pw1, dw1);
-        } else {
-            auto generic_half = [&](int hf) __attribute__((always_inline)) {
-                const int ih0 = i0 + 32 * hf;
-                if (!half_active(ih0)) return;
-                f32x16_t s[KB], dp[KB];
-                uint32_t pw[KB][8], dw[KB][8];
-                half_sp(qt, gt, lse_t + 32 * hf, delta_t + 32 * hf, hf, s, dp);
-                if (!half_needs_mask(ih0))
-                    half_exp(s, lse_t + 32 * hf, ih0, std::integral_constant<int, 0>{});
-                else if (a.window > 0)
-                    half_exp(s, lse_t + 32 * hf, ih0, std::integral_constant<int, 2>{});
-                else
-                    half_exp(s, lse_t + 32 * hf, ih0, std::integral_constant<int, 1>{});
-                half_ds(s, dp, delta_t + 32 * hf, mask_t + 32 * hf, ih0, pw, dw);
-                half_out(qt, gt, hf, pw, dw);
-            };
-            generic_half(0);
-            generic_half(1);
+        // Where two workgroups share a CU the request is issued in the middle, once the score
+        // registers of the first half are dead, which keeps the staging registers out of the
+        // busiest stretch.
+        constexpr bool kLateRequest = DPAD <= 64;
+        if constexpr (!kLateRequest) request_tile(regs, t + 1);
+        std::integral_constant<int, 0> none;
+        f32x16_t s0[KB], s1[KB], p0[KB], p1[KB];
+        uint32_t pw0[KB][8], dw0[KB][8], pw1[KB][8], dw1[KB][8];
+        half_sp(qt, gt, lse_t, delta_t, 0, s0, p0);
+        half_exp(s0, lse_t, i0, none);
+        half_sp(qt, gt, lse_t + 32, delta_t + 32, 1, s1, p1);
+        half_ds(s0, p0, delta_t, mask_t, i0, pw0, dw0);
+        half_exp(s1, lse_t + 32, i0 + 32, none);
+        if constexpr (kLateRequest) {
+            __builtin_amdgcn_sched_barrier(0);
+            request_tile(regs, t + 1);
+            __builtin_amdgcn_sched_barrier(0);
         }
+        half_out(qt, gt, 0, pw0, dw0);
+        half_ds(s1, p1, delta_t + 32, mask_t + 32, i0 + 32, pw1, dw1);
+        half_out(qt, gt, 1, pw1, dw1);
         // stage the next query tile (its buffer was last read before the previous barrier)
-        if (have_next) {
-            qst.fix(i0 + kBwdBM, a.sq, a.d);
-            gst.fix(i0 + kBwdBM, a.sq, a.d);
-            qst.store(q_lds + (buf ^ 1) * SM::kQTile);
-            gst.store(g_lds + (buf ^ 1) * SM::kQTile);
-            store_stats(buf ^ 1, i0 + kBwdBM);
-            store_mask(buf ^ 1);
-        }
+        if (t + 1 < t_hi) stage_tile(regs, t + 1);
         __syncthreads();
     };
-    auto tile_fast = [&](int t) __attribute__((always_inline)) {
-        const int i0 = t * kBwdBM;
-        return a.window <= 0 && k0 + kBN <= a.sk && i0 + kBwdBM <= a.sq &&
-               (!a.causal || i0 >= k0 + kBN - 1);
+
+    // Diagonal / window / tail tiles: activity and masks are tested per wavefront and half tile.
+    // The half tiles of `n` tiles (1 or 2) that sit in LDS are walked by one rolled loop.
+    auto generic_tiles = [&](int t, int n) __attribute__((always_inline)) {
+#pragma unroll 1
+        for (int j = 0; j < 2 * n; ++j) {
+            const int tt = t + (j >> 1), hf = j & 1;
+            const int ih0 = tt * kBwdBM + 32 * hf;
+            if (!half_active(ih0)) continue;
+            const int buf = (tt - t_lo) & 1;
+            const T* qt = q_lds + buf * SM::kQTile;
+            const T* gt = g_lds + buf * SM::kQTile;
+            const float* lse_h = stat_lds + buf * 2 * kBwdBM + 32 * hf;
+            const float* delta_h = lse_h + kBwdBM;
+            const uint32_t* mask_h = mask_lds + buf * kBwdThreads + wave * kBwdBM + 32 * hf;
+            f32x16_t s[KB], dp[KB];
+            uint32_t pw[KB][8], dw[KB][8];
+            half_sp(qt, gt, lse_h, delta_h, hf, s, dp);
+            if (!half_needs_mask(ih0))
+                half_exp(s, lse_h, ih0, std::integral_constant<int, 0>{});
+            else if (a.window > 0)
+                half_exp(s, lse_h, ih0, std::integral_constant<int, 2>{});
+            else
+                half_exp(s, lse_h, ih0, std::integral_constant<int, 1>{});
+            half_ds(s, dp, delta_h, mask_h, ih0, pw, dw);
+            half_out(qt, gt, hf, pw, dw);
+        }
+    };
+    // Generic step at tile t (in LDS, nothing requested); returns the number of tiles done.  Two
+    // generic tiles in a row -- the two diagonal tiles of a causal mask -- are taken together:
+    // the wavefronts have very different numbers of visible half tiles in each of them, and with
+    // both tiles in LDS no wavefront waits at a barrier in between for the busiest one.
+    auto generic_step = [&](int t) __attribute__((always_inline)) -> int {
+        const bool pair = kPairGeneric && t + 1 < t_hi && !tile_fast(t + 1);
+        if (!pair) {
+            request_tile(regs, t + 1);
+            generic_tiles(t, 1);
+            if (t + 1 < t_hi) stage_tile(regs, t + 1);
+            __syncthreads();
+            return 1;
+        }
+        if (!(pair_first && t == t_lo)) {  // otherwise the start-up has staged tile t+1 already
+            request_tile(regs, t + 1);
+            stage_tile(regs, t + 1);  // the other buffer: last read before the previous barrier
+            __syncthreads();
+        }
+        request_tile(regs, t + 2);
+        generic_tiles(t, 2);
+        __syncthreads();  // tile t+2 goes where tile t was
+        if (t + 2 < t_hi) stage_tile(regs, t + 2);
+        __syncthreads();
+        return 2;
     };
     {
         int t = t_lo;
-        for (; t < t_hi && !tile_fast(t); ++t) iteration(t, std::false_type{});
-        for (; t < t_hi && tile_fast(t); ++t) iteration(t, std::true_type{});
-        for (; t < t_hi; ++t) iteration(t, std::false_type{});
+        while (t < t_hi && !tile_fast(t)) t += generic_step(t);
+        for (; t < t_hi && tile_fast(t); ++t) fast_iteration(t);
+        while (t < t_hi) t += generic_step(t);
     }
     // ---- write dK, dV ----
 #pragma unroll
