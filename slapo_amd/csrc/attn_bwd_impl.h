@@ -465,7 +465,14 @@ __global__ __launch_bounds__(kBwdThreads, ((DPAD <= 64 && KB == 1) ? 2 : 1)) voi
 
     // Fast iteration t (every key of the workgroup sees every query of the tile): request tile
     // t+1, process tile t as one straight block, write tile t+1 into the other buffer.
-    auto fast_iteration = [&](int t) __attribute__((always_inline)) {
+    // The two halves of tile t with their stages staggered (mask_tag as in half_exp; only fast
+    // tiles, tag 0, run this body: a second copy with the causal bound for the diagonal tiles
+    // changed the register allocation of the first and measured 6 % slower overall).
+    // kRequestInside: tile t+1 is requested in the middle, once the score registers of the first
+    // half are dead, which keeps the staging registers out of the busiest stretch.
+    auto staggered_tile = [&](int t, auto mask_tag, auto request_inside)
+                              __attribute__((always_inline)) {
+        constexpr bool kRequestInside = decltype(request_inside)::value;
         const int buf = (t - t_lo) & 1;
         const T* qt = q_lds + buf * SM::kQTile;
         const T* gt = g_lds + buf * SM::kQTile;
@@ -473,20 +480,14 @@ __global__ __launch_bounds__(kBwdThreads, ((DPAD <= 64 && KB == 1) ? 2 : 1)) voi
         const float* delta_t = lse_t + kBwdBM;
         const uint32_t* mask_t = mask_lds + buf * kBwdThreads + wave * kBwdBM;
         const int i0 = t * kBwdBM;
-        // Where two workgroups share a CU the request is issued in the middle, once the score
-        // registers of the first half are dead, which keeps the staging registers out of the
-        // busiest stretch.
-        constexpr bool kLateRequest = DPAD <= 64;
-        if constexpr (!kLateRequest) request_tile(regs, t + 1);
-        std::integral_constant<int, 0> none;
         f32x16_t s0[KB], s1[KB], p0[KB], p1[KB];
         uint32_t pw0[KB][8], dw0[KB][8], pw1[KB][8], dw1[KB][8];
         half_sp(qt, gt, lse_t, delta_t, 0, s0, p0);
-        half_exp(s0, lse_t, i0, none);
+        half_exp(s0, lse_t, i0, mask_tag);
         half_sp(qt, gt, lse_t + 32, delta_t + 32, 1, s1, p1);
         half_ds(s0, p0, delta_t, mask_t, i0, pw0, dw0);
-        half_exp(s1, lse_t + 32, i0 + 32, none);
-        if constexpr (kLateRequest) {
+        half_exp(s1, lse_t + 32, i0 + 32, mask_tag);
+        if constexpr (kRequestInside) {
             __builtin_amdgcn_sched_barrier(0);
             request_tile(regs, t + 1);
             __builtin_amdgcn_sched_barrier(0);
@@ -494,6 +495,14 @@ __global__ __launch_bounds__(kBwdThreads, ((DPAD <= 64 && KB == 1) ? 2 : 1)) voi
         half_out(qt, gt, 0, pw0, dw0);
         half_ds(s1, p1, delta_t + 32, mask_t + 32, i0 + 32, pw1, dw1);
         half_out(qt, gt, 1, pw1, dw1);
+    };
+    // Fast iteration t (every key of the workgroup sees every query of the tile): request tile
+    // t+1, process tile t as one straight block, write tile t+1 into the other buffer.
+    auto fast_iteration = [&](int t) __attribute__((always_inline)) {
+        constexpr bool kLateRequest = DPAD <= 64;  // two workgroups share a CU: registers scarce
+        if constexpr (!kLateRequest) request_tile(regs, t + 1);
+        staggered_tile(t, std::integral_constant<int, 0>{},
+                       std::integral_constant<bool, kLateRequest>{});
         // stage the next query tile (its buffer was last read before the previous barrier)
         if (t + 1 < t_hi) stage_tile(regs, t + 1);
         __syncthreads();
