@@ -55,7 +55,7 @@ def _check(q, k, v, do, mask, causal, window, dtype, p=0.0):
         assert_parity(a, r, dtype, name)
 
 
-# ---- BASELINE configs at reduced batch / heads (the oracle must finish in seconds) ----------
+# ---- the benchmark configurations at reduced batch / heads (the oracle must finish in seconds)
 def test_cfg1_bert_large_fp32_forward():
     """fp32, S 512, 16 heads x 64, no mask, forward (batch 1 of the 4)."""
     q, k, v, do, _ = _inputs(1, 512, 16, 64, torch.float32)
@@ -267,7 +267,7 @@ def test_argument_errors():
         op.hip_attention(odd, odd, odd)
 
 
-# ---- full BASELINE sizes through size-independent properties -----------------------------------
+# ---- full benchmark sizes through size-independent properties ---------------------------------
 def test_full_size_cfg2_properties():
     """fp16, B 8, S 1024, 16 x 64, causal, at full size: (1) V = const gives that const back
     (rows of P sum to one); (2) query 0 returns V[0]; (3) linearity in V; (4) agreement with the

@@ -132,5 +132,5 @@ def test_attended_pairs_formulas():
     assert OA.attended_pairs(s, s, True, w) == w * (w + 1) // 2 + (s - w) * w
     L = 40
     assert OA.attended_pairs(s, s, True, 0, L) == L * (L + 1) // 2 + (s - L) * L
-    # BASELINE figure for GPT-2-medium shape: 524800 pairs per head at S = 1024
+    # the GPT-2-medium benchmark shape: 524800 pairs per head at S = 1024
     assert OA.attended_pairs(1024, 1024, True) == 524800
