@@ -62,6 +62,8 @@ class _HipAttention(torch.autograd.Function):
         b, sq, h, _ = q.shape
         sk = k.shape[1]
         plan, seed, offset = None, 0, 0
+        if b * h * sq * sk == 0:
+            p = 0.0  # nothing to drop, and F.dropout leaves the generator alone for an empty tensor
         if p > 0.0:
             plan = K.dropout_plan(b * h * sq * sk, 4, q.device)
             if p < 1.0:

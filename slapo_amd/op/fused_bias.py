@@ -50,6 +50,8 @@ class _BiasDropoutResidual(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, bias, residual, p):
         plan, seed, offset = None, 0, 0
+        if x.numel() == 0:
+            p = 0.0  # nothing to drop, and F.dropout leaves the generator alone for an empty tensor
         if 0.0 < p:
             plan = K.dropout_plan(x.numel(), x.element_size(), x.device)
             if p < 1.0:
@@ -96,6 +98,8 @@ class _BiasDropoutResidualLayerNorm(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x, bias, residual, weight, ln_bias, p, eps):
         plan, seed, offset = None, 0, 0
+        if x.numel() == 0:
+            p = 0.0  # nothing to drop, and F.dropout leaves the generator alone for an empty tensor
         if 0.0 < p:
             plan = K.dropout_plan(x.numel(), x.element_size(), x.device)
             if p < 1.0:
