@@ -20,12 +20,40 @@ def _require_device(*tensors):
             )
 
 
+# The wrappers below sit on the critical path of every training step, so the per-call host work
+# is kept small: raw stream and data pointers as plain integers (ctypes converts them through the
+# declared argtypes), a device switch only when the tensor lives on another device than the
+# current one, and parameter structs cached per problem geometry.
 def _stream():
-    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    return torch._C._cuda_getCurrentRawStream(torch.cuda.current_device())
 
 
 def _ptr(t):
-    return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
+    return t.data_ptr() if t is not None else None
+
+
+class _on:
+    """`with _on(device):` -- like torch.cuda.device(device), without the cost when the device
+    is already current."""
+
+    __slots__ = ("idx", "prev")
+
+    def __init__(self, device):
+        self.idx = torch.device(device).index
+        self.prev = -1
+
+    def __enter__(self):
+        if self.idx is not None:
+            cur = torch.cuda.current_device()
+            if cur != self.idx:
+                self.prev = cur
+                torch.cuda.set_device(self.idx)
+        return self
+
+    def __exit__(self, *exc):
+        if self.prev >= 0:
+            torch.cuda.set_device(self.prev)
+        return False
 
 
 @functools.lru_cache(maxsize=4096)
@@ -64,7 +92,7 @@ def bias_gelu_fwd(y, bias):
     out = torch.empty_like(y)
     if y.numel() == 0:
         return out
-    with torch.cuda.device(y.device):
+    with _on(y.device):
         rc = _lib.load().slapo_amd_bias_gelu_fwd(_ptr(y), _ptr(bias), _ptr(out), rows, cols,
                                                  _lib.dtype_code(y.dtype), _stream())
     _lib.check(rc, "slapo_amd_bias_gelu_fwd")
@@ -85,7 +113,7 @@ def bias_gelu_bwd(grad, y, bias, need_dbias=True):
     dbias = torch.empty_like(bias) if need_dbias else None
     if y.numel() == 0:
         return dx, (dbias.zero_() if dbias is not None else None)
-    with torch.cuda.device(y.device):
+    with _on(y.device):
         ws, nbytes = _colsum_ws(rows, cols, y.device) if need_dbias else (None, 0)
         rc = _lib.load().slapo_amd_bias_gelu_bwd(_ptr(grad), _ptr(y), _ptr(bias), _ptr(dx),
                                                  _ptr(dbias), _ptr(ws), nbytes, rows, cols,
@@ -105,7 +133,7 @@ def bias_dropout_residual_fwd(x, bias, residual, p, seed, offset, plan):
     out = torch.empty_like(x)
     if x.numel() == 0:
         return out
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         rc = _lib.load().slapo_amd_bias_dropout_residual_fwd(
             _ptr(x), _ptr(bias), _ptr(residual), _ptr(out), rows, cols,
             _lib.dtype_code(x.dtype), float(p), seed, offset,
@@ -124,7 +152,7 @@ def bias_dropout_residual_bwd(grad, bias_like, p, seed, offset, plan, need_dx=Tr
     dbias = torch.empty(cols, dtype=grad.dtype, device=grad.device) if need_dbias else None
     if grad.numel() == 0 or not (need_dx or need_dbias):
         return dx, (dbias.zero_() if dbias is not None else None)
-    with torch.cuda.device(grad.device):
+    with _on(grad.device):
         ws, nbytes = _colsum_ws(rows, cols, grad.device) if need_dbias else (None, 0)
         rc = _lib.load().slapo_amd_bias_dropout_residual_bwd(
             _ptr(grad), _ptr(dx), _ptr(dbias), _ptr(ws), nbytes, rows, cols,
@@ -160,7 +188,7 @@ def bias_dropout_residual_ln_fwd(x, bias, residual, weight, ln_bias, eps, p, see
         rstd = torch.empty(rows, dtype=torch.float32, device=x.device)
     if x.numel() == 0:
         return y, z, mean, rstd
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         rc = _lib.load().slapo_amd_bias_dropout_residual_ln_fwd(
             _ptr(x), _ptr(bias), _ptr(residual), _ptr(weight), _ptr(ln_bias), _ptr(z), _ptr(y),
             _ptr(mean), _ptr(rstd), rows, cols, _lib.dtype_code(x.dtype), float(eps), float(p),
@@ -189,7 +217,7 @@ def bias_dropout_residual_ln_bwd(grad, z, mean, rstd, weight, p, seed, offset, p
                 o.zero_()
         return outs
     lib = _lib.load()
-    with torch.cuda.device(z.device):
+    with _on(z.device):
         ws, nbytes = None, 0
         if need_dweight or need_dln_bias or need_dbias:
             nbytes = lib.slapo_amd_ln_bwd_workspace_bytes(rows, cols)
@@ -214,7 +242,7 @@ def vocab_ce_fwd(logits, target, vocab_start=0):
         raise ValueError("target must have the shape of the logits without the vocabulary dim")
     stats = torch.empty(4, max(rows, 1), dtype=torch.float32, device=logits.device)
     if rows:
-        with torch.cuda.device(logits.device):
+        with _on(logits.device):
             rc = _lib.load().slapo_amd_vocab_ce_fwd(
                 _ptr(logits), _ptr(target), _ptr(stats[0]), _ptr(stats[1]), _ptr(stats[2]),
                 _ptr(stats[3]), rows, vocab, int(vocab_start), _lib.dtype_code(logits.dtype),
@@ -231,7 +259,7 @@ def vocab_ce_bwd(logits, target, row_max, inv_sum_exp, grad_loss, vocab_start=0,
     grad = torch.empty_like(logits)
     grad_loss = grad_loss.contiguous().view(-1).float()
     if rows:
-        with torch.cuda.device(logits.device):
+        with _on(logits.device):
             rc = _lib.load().slapo_amd_vocab_ce_bwd(
                 _ptr(logits), _ptr(target), _ptr(row_max.contiguous()),
                 _ptr(inv_sum_exp.contiguous()), _ptr(grad_loss), _ptr(grad), rows, vocab,
@@ -245,7 +273,7 @@ def dropout_mask(numel, elem_bytes, p, seed, offset, device):
     """Boolean keep-mask [numel] drawn on the device (debugging / test aid)."""
     plan = dropout_plan(numel, elem_bytes, device)
     mask = torch.empty(numel, dtype=torch.uint8, device=device)
-    with torch.cuda.device(device):
+    with _on(device):
         rc = _lib.load().slapo_amd_dropout_mask(_ptr(mask), ctypes.byref(plan), float(p), seed,
                                                 offset, _stream())
     _lib.check(rc, "slapo_amd_dropout_mask")
@@ -255,12 +283,18 @@ def dropout_mask(numel, elem_bytes, p, seed, offset, device):
 # ------------------------------------------------------------------------------------------
 # attention
 # ------------------------------------------------------------------------------------------
+@functools.lru_cache(maxsize=1024)
+def _stride_array(s0, s1, s2):
+    return (ctypes.c_int64 * 3)(s0, s1, s2)
+
+
 def _bshd_strides(t):
     if t.ndim != 4:
         raise ValueError("attention operands must be [batch, seqlen, heads, head_dim]")
-    if t.shape[-1] > 1 and t.stride(-1) != 1:
+    st = t.stride()
+    if t.shape[-1] > 1 and st[3] != 1:
         raise ValueError("head_dim must be contiguous")
-    return (ctypes.c_int64 * 3)(t.stride(0), t.stride(1), t.stride(2))
+    return _stride_array(st[0], st[1], st[2])
 
 
 def _usable_layout(t):
@@ -273,26 +307,41 @@ def _usable_layout(t):
     return t
 
 
+_PARAMS_CACHE = {}
+
+
 def make_attn_params(q, k, v, o, bias, causal, window, scale, p, seed, offset, plan,
                      keep_mask=None):
-    prm = AttnParams()
-    b, sq, h, d = q.shape
-    prm.dtype = _lib.dtype_code(q.dtype)
-    prm.batch, prm.heads, prm.seqlen_q, prm.seqlen_k, prm.head_dim = b, h, sq, k.shape[1], d
-    prm.causal = 1 if causal else 0
-    prm.window = int(window) if window else 0
-    prm.scale = float(scale)
-    prm.p_drop = float(p)
+    """The parameter struct of one attention call.  Everything but (seed, offset, keep_mask) is a
+    function of the problem geometry and is cached."""
+    key = (q.dtype, q.shape, k.shape[1], q.stride(), k.stride(), v.stride(), o.stride(),
+           bias.stride() if bias is not None else None, bool(causal), int(window or 0),
+           float(scale), float(p), id(plan))
+    entry = _PARAMS_CACHE.get(key)
+    if entry is None:
+        prm = AttnParams()
+        b, sq, h, d = q.shape
+        prm.dtype = _lib.dtype_code(q.dtype)
+        prm.batch, prm.heads, prm.seqlen_q, prm.seqlen_k, prm.head_dim = b, h, sq, k.shape[1], d
+        prm.causal = 1 if causal else 0
+        prm.window = int(window) if window else 0
+        prm.scale = float(scale)
+        prm.p_drop = float(p)
+        prm.q_strides = _bshd_strides(q)
+        prm.k_strides = _bshd_strides(k)
+        prm.v_strides = _bshd_strides(v)
+        prm.o_strides = _bshd_strides(o)
+        if bias is not None:
+            prm.bias_strides = (ctypes.c_int64 * 4)(*bias.stride())
+        if plan is not None:
+            prm.plan = plan
+        if len(_PARAMS_CACHE) >= 1024:
+            _PARAMS_CACHE.clear()
+        # the plan object is kept alive with the entry, so that its id stays unique
+        entry = _PARAMS_CACHE[key] = (prm, plan)
+    prm = AttnParams.from_buffer_copy(entry[0])
     prm.seed = int(seed)
     prm.offset = int(offset)
-    prm.q_strides = _bshd_strides(q)
-    prm.k_strides = _bshd_strides(k)
-    prm.v_strides = _bshd_strides(v)
-    prm.o_strides = _bshd_strides(o)
-    if bias is not None:
-        prm.bias_strides = (ctypes.c_int64 * 4)(*bias.stride())
-    if plan is not None:
-        prm.plan = plan
     if keep_mask is not None:
         prm.keep_mask = keep_mask.data_ptr()
     return prm
@@ -325,7 +374,7 @@ def attn_fwd(q, k, v, bias, causal, window, scale, p, seed, offset, plan, save_m
             keep_mask = torch.empty(nbytes // 4, dtype=torch.int32, device=q.device)
             prm.keep_mask = keep_mask.data_ptr()
     if o.numel():
-        with torch.cuda.device(q.device):
+        with _on(q.device):
             rc = _lib.load().slapo_amd_attn_fwd(ctypes.byref(prm), _ptr(q), _ptr(k), _ptr(v),
                                                 _ptr(bias), _ptr(o), _ptr(lse), _stream())
         _lib.check(rc, "slapo_amd_attn_fwd")
@@ -348,7 +397,7 @@ def attn_bwd(dout, q, k, v, bias, o, lse, causal, window, scale, p, seed, offset
     if dq.numel() and dk.numel():
         lib = _lib.load()
         nbytes = lib.slapo_amd_attn_bwd_workspace_bytes(ctypes.byref(prm))
-        with torch.cuda.device(q.device):
+        with _on(q.device):
             ws = torch.empty(max(nbytes // 4, 1), dtype=torch.float32, device=q.device)
             rc = lib.slapo_amd_attn_bwd(
                 ctypes.byref(prm), _ptr(q), _ptr(k), _ptr(v), _ptr(bias), _ptr(o), _ptr(dout),
