@@ -49,6 +49,9 @@ def warning_once(msg):
 # them instead of regenerating every Philox block in both of its kernels.  Same gradients, bit
 # for bit; False trades the buffer (B*H*Sq*Sk/8 bytes) for the regeneration.
 SAVE_DROPOUT_MASK = True
+# ... up to this size per call; beyond it (long sequences: the bits grow with Sq * Sk) the backward
+# regenerates the mask and nothing of that size is kept between the passes.
+SAVE_DROPOUT_MASK_MAX_BYTES = 512 << 20
 
 
 class _HipAttention(torch.autograd.Function):
@@ -69,6 +72,9 @@ class _HipAttention(torch.autograd.Function):
             if p < 1.0:
                 seed, offset = draw_philox(plan.offset_increment, q.device)
         save_mask = SAVE_DROPOUT_MASK and 0.0 < p < 1.0 and any(ctx.needs_input_grad[:3])
+        if save_mask:
+            mask_bytes = b * h * ((sk + 31) // 32) * ((sq + 3) // 4 * 4) * 4
+            save_mask = mask_bytes <= SAVE_DROPOUT_MASK_MAX_BYTES
         out, lse, (q, k, v), keep_mask = K.attn_fwd(q, k, v, bias, causal, window, scale, p, seed,
                                                     offset, plan, save_mask=save_mask)
         ctx.save_for_backward(q, k, v, bias, out, lse, keep_mask)

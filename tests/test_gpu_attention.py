@@ -201,6 +201,14 @@ def test_dropout_keep_bits_saved_by_the_forward(dtype, shape, causal, window, ma
         A.SAVE_DROPOUT_MASK = True
     for a, r in zip(with_bits, regenerated):
         assert torch.equal(a, r)
+    cap = A.SAVE_DROPOUT_MASK_MAX_BYTES
+    A.SAVE_DROPOUT_MASK_MAX_BYTES = 0  # a buffer above the cap is not kept either
+    try:
+        capped = _run(q, k, v, do, mask, causal, window, p)
+    finally:
+        A.SAVE_DROPOUT_MASK_MAX_BYTES = cap
+    for a, r in zip(with_bits, capped):
+        assert torch.equal(a, r)
 
     # the buffer itself: every word that the forward visits holds torch's mask bits
     qd, kd, vd = q.cuda(), k.cuda(), v.cuda()
