@@ -304,11 +304,15 @@ def main():
     for _ in range(args.warmup):
         step.step()
     torch.cuda.synchronize()
+    # Per-kernel durations come from HIP events around the three launches of every fourth step of
+    # the timed region: an event between two kernels costs about 1 us of stream time, which at
+    # 150 us per step would show in `value` if every step carried four of them.
+    every = 4
     events = [[torch.cuda.Event(enable_timing=True) for _ in range(4)]
-              for _ in range(args.steps)]
+              for _ in range((args.steps + every - 1) // every)]
     t0 = time.perf_counter()
     for i in range(args.steps):
-        step.step(events[i])
+        step.step(events[i // every] if i % every == 0 else None)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
 
@@ -316,7 +320,7 @@ def main():
     d = cfg["head_dim"]
     ms_per_step = elapsed / args.steps * 1e3
     value = 14 * d * n_pairs / (elapsed / args.steps) / 1e12
-    seg_ms = [sum(ev[i].elapsed_time(ev[i + 1]) for ev in events) / args.steps for i in range(3)]
+    seg_ms = [sum(ev[i].elapsed_time(ev[i + 1]) for ev in events) / len(events) for i in range(3)]
     kern_ms = seg_ms[2]
     bwd_flops = 8 * d * n_pairs
     achieved = bwd_flops / (kern_ms * 1e-3) / 1e12
