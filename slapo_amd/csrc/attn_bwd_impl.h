@@ -44,11 +44,17 @@ struct BwdSmem {
     static constexpr size_t kBytes = 2 * kQBytes + kStatBytes + kMaskBytes;
 };
 
+constexpr bool bwd_two_per_cu(int dpad, int drop, int kb) {
+    return kb == 1 && (dpad <= 64 || (dpad == 96 && drop != 3));
+}
+
 // KB = blocks of 32 keys per wavefront.  KB = 2 halves the LDS operand traffic per matrix
 // instruction (every Q / dO fragment read feeds two MFMAs) at the price of twice the resident
 // fragments and accumulators, i.e. one wavefront per SIMD instead of two.
 template <typename T, int DPAD, bool kBias, int kDrop, int KB>
-__global__ __launch_bounds__(kBwdThreads, ((DPAD <= 64 && KB == 1) ? 2 : 1)) void attn_bwd_kernel(
+// Two workgroups per CU up to DPAD 96, one at 128 (192 resident accumulator / fragment registers)
+// and at 96 with the forward's keep bits (measured 23-35 % slower with two than with one).
+__global__ __launch_bounds__(kBwdThreads, (bwd_two_per_cu(DPAD, kDrop, KB) ? 2 : 1)) void attn_bwd_kernel(
     const AttnArgs a) {
     static_assert(kDrop != 3 || KB == 1, "the keep-bit tile holds one word per wavefront and query");
     typedef typename Mma<T>::frag frag_t;
@@ -463,6 +469,29 @@ __global__ __launch_bounds__(kBwdThreads, ((DPAD <= 64 && KB == 1) ? 2 : 1)) voi
         }
     };
 
+    // The two halves of a fast tile one after the other.  At DPAD 96 this is what fits two
+    // workgroups per CU (11-51 spilled registers); the second resident workgroup is worth more
+    // than the stagger: 319 -> 287 us at bf16 B4 S2048 H32 D80 causal, 638 -> 503 us when the
+    // backward regenerates the dropout mask.  With the forward's keep bits it is the other way
+    // round (370 -> 455 us), so that variant keeps one workgroup and the staggered body.
+    auto sequential_tile = [&](int t) __attribute__((always_inline)) {
+        const int buf = (t - t_lo) & 1;
+        const T* qt = q_lds + buf * SM::kQTile;
+        const T* gt = g_lds + buf * SM::kQTile;
+#pragma unroll
+        for (int hf = 0; hf < 2; ++hf) {
+            const int ih0 = t * kBwdBM + 32 * hf;
+            const float* lse_h = stat_lds + buf * 2 * kBwdBM + 32 * hf;
+            const float* delta_h = lse_h + kBwdBM;
+            const uint32_t* mask_h = mask_lds + buf * kBwdThreads + wave * kBwdBM + 32 * hf;
+            f32x16_t s[KB], dp[KB];
+            uint32_t pw[KB][8], dw[KB][8];
+            half_sp(qt, gt, lse_h, delta_h, hf, s, dp);
+            half_exp(s, lse_h, ih0, std::integral_constant<int, 0>{});
+            half_ds(s, dp, delta_h, mask_h, ih0, pw, dw);
+            half_out(qt, gt, hf, pw, dw);
+        }
+    };
     // Fast iteration t (every key of the workgroup sees every query of the tile): request tile
     // t+1, process tile t as one straight block, write tile t+1 into the other buffer.
     // The two halves of tile t with their stages staggered (mask_tag as in half_exp; only fast
@@ -501,7 +530,10 @@ __global__ __launch_bounds__(kBwdThreads, ((DPAD <= 64 && KB == 1) ? 2 : 1)) voi
     auto fast_iteration = [&](int t) __attribute__((always_inline)) {
         constexpr bool kLateRequest = DPAD <= 64;  // two workgroups share a CU: registers scarce
         if constexpr (!kLateRequest) request_tile(regs, t + 1);
-        staggered_tile(t, std::integral_constant<int, 0>{},
+        if constexpr (DPAD == 96 && bwd_two_per_cu(DPAD, kDrop, KB))
+            sequential_tile(t);
+        else
+            staggered_tile(t, std::integral_constant<int, 0>{},
                        std::integral_constant<bool, kLateRequest>{});
         // stage the next query tile (its buffer was last read before the previous barrier)
         if (t + 1 < t_hi) stage_tile(regs, t + 1);
