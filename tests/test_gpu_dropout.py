@@ -127,3 +127,56 @@ def test_recompute_under_restored_state_reproduces_mask():
     assert torch.equal(a, b) and _gen().get_offset() == moved
     c = op.hip_attention(q, k, v, None, causal=True, p=0.3)
     assert not torch.equal(a, c)
+
+
+def test_checkpointed_block_of_hip_ops_matches_the_plain_run():
+    """Activation checkpointing with tracked streams around the HIP ops (reference
+    slapo/checkpoint.py:15-124, tests/test_checkpoint.py:138-198): attention dropout under the
+    forked stream, the fused epilogues under the outer one.  Output and every gradient of the
+    checkpointed run equal the plain run bit for bit, and the recompute leaves both streams
+    where the forward left them."""
+    import slapo_amd
+    from slapo_amd.checkpoint import checkpoint
+    from slapo_amd.random import get_cuda_rng_tracker
+
+    B, S, H, D = 2, 256, 4, 64
+    hid = H * D
+    dt = torch.float16
+    g = torch.Generator(device="cuda").manual_seed(1)
+    qkv_w = (torch.randn(hid, 3 * hid, device="cuda", dtype=dt, generator=g) * 0.05).requires_grad_()
+    out_b = torch.randn(hid, device="cuda", dtype=dt, generator=g).requires_grad_()
+    ln = op.HipBiasDropoutResidualLayerNorm(hid, p=0.2, device="cuda", dtype=dt)
+    up_b = torch.randn(hid, device="cuda", dtype=dt, generator=g).requires_grad_()
+    x0 = torch.randn(B, S, hid, device="cuda", dtype=dt, generator=g)
+    params = [qkv_w, out_b, up_b, ln.weight, ln.bias]
+
+    def block(x, p_attn):
+        qkv = (x @ qkv_w).view(B, S, H, 3 * D)
+        q, k, v = qkv.split(D, dim=-1)             # strided views, read in place
+        with get_cuda_rng_tracker().fork():
+            a = op.hip_attention(q, k, v, None, causal=True, p=p_attn)
+        h = ln(a.reshape(B, S, hid), out_b, x)
+        h = op.bias_gelu(h, up_b)
+        return op.bias_dropout_residual(h, out_b, x, 0.1, True)
+
+    def run(use_checkpoint):
+        slapo_amd.set_random_seed(123, None, None, 0)
+        x = x0.clone().requires_grad_()
+        out = checkpoint(block, x, 0.3) if use_checkpoint else block(x, 0.3)
+        offset = _gen().get_offset()
+        forked = get_cuda_rng_tracker().get_states()["model-parallel-rng"].clone()
+        assert offset > 0
+        out.float().square().mean().backward()
+        assert _gen().get_offset() == offset
+        assert torch.equal(get_cuda_rng_tracker().get_states()["model-parallel-rng"], forked)
+        grads = [t.grad.clone() for t in [x] + params]
+        for t in params:
+            t.grad = None
+        return [out.detach()] + grads
+
+    ref = run(False)
+    got = run(True)
+    for a, b in zip(ref, got):
+        assert torch.equal(a, b)
+    assert ref[0].isfinite().all() and (ref[1] != 0).any()
+    get_cuda_rng_tracker().reset()

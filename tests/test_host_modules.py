@@ -226,3 +226,64 @@ def test_set_random_seed_arithmetic():
     a = torch.rand(3)
     slapo_amd.set_random_seed(2013, dp_rank=3, pp_rank=2)
     torch.testing.assert_close(torch.rand(3), a)
+
+
+def test_checkpoint_replays_every_random_stream(monkeypatch):
+    """The reference's test of its checkpoint with forked streams
+    (tests/test_checkpoint.py:138-198), on the host: a block that draws from the outer stream,
+    from the forked stream and from the host generator gives the same output and gradients with
+    and without the checkpoint, and the recompute moves none of the streams."""
+    import importlib
+    ckpt = importlib.import_module("slapo_amd.checkpoint")  # the package attribute is the function
+
+    be = _FakeBackend()
+    tr = CudaRNGStatesTracker(be)
+    monkeypatch.setattr(ckpt, "get_cuda_rng_tracker", lambda: tr)
+    monkeypatch.setattr(ckpt, "is_random_seed_set", lambda: bool(tr.get_states()))
+
+    def device_dropout(x):
+        seed, off = be.draw()
+        g = torch.Generator().manual_seed(seed * 1000 + off)
+        return x * (torch.rand(x.shape, generator=g) < 0.5) * 2.0
+
+    w1 = torch.randn(6, 5, requires_grad=True)
+    w2 = torch.randn(5, 6, requires_grad=True)
+    calls = []
+
+    def block(x, tag):
+        calls.append(tag)
+        h = x @ w1
+        with tr.fork():
+            h = device_dropout(h)
+        h = device_dropout(h @ w2)
+        return nn.functional.dropout(h, 0.5)  # host generator
+
+    def run(use_checkpoint):
+        be.manual_seed(123)
+        tr.reset()
+        tr.add("model-parallel-rng", 123 + 2718)
+        torch.manual_seed(5)
+        x = torch.arange(36.0).reshape(6, 6).requires_grad_()
+        out = ckpt.checkpoint(block, x, "t") if use_checkpoint else block(x, "t")
+        before = (be.state, tr.get_states(), torch.get_rng_state())
+        out.mean().backward()
+        after = (be.state, tr.get_states(), torch.get_rng_state())
+        assert before[0] == after[0] and before[1] == after[1] and torch.equal(before[2], after[2])
+        grads = [t.grad.clone() for t in (x, w1, w2)]
+        w1.grad = w2.grad = None
+        return [out.detach()] + grads
+
+    ref = run(False)
+    n = len(calls)
+    got = run(True)
+    assert len(calls) == n + 2 and calls[-1] == "t"   # forward and one recompute
+    for a, b in zip(ref, got):
+        assert torch.equal(a, b)
+    assert be.state == (123, 4) and tr.get_states()["model-parallel-rng"] == (123 + 2718, 4)
+
+    # without tracked streams the call goes to torch's own checkpoint
+    tr.reset()
+    x = torch.randn(6, 6, requires_grad=True)
+    out = ckpt.checkpoint(lambda t: (t @ w1).relu(), x, use_reentrant=False)
+    out.sum().backward()
+    assert x.grad is not None and w1.grad is not None
