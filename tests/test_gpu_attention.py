@@ -179,6 +179,7 @@ def test_dropout_mask_bits_read_back_exactly():
     ((1, 320, 2, 128), True, 0, False, 0.1),    # sequential halves, two workgroups per CU
     ((1, 320, 2, 128), True, 100, False, 0.1),  # local window (staggered variant at 128)
     ((1, 192, 2, 80), False, 0, True, 0.2),     # head_dim 80 (padded to 96)
+    ((1, 320, 2, 80), True, 0, False, 0.1),     # ... causal: sequential and diagonal tile bodies
 ])
 def test_dropout_keep_bits_saved_by_the_forward(dtype, shape, causal, window, masked, p):
     """The forward stores the keep bits, the backward reads them: gradients are bitwise those of
