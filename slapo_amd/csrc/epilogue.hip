@@ -442,16 +442,19 @@ __global__ __launch_bounds__(256) void bias_dropout_residual_ln_fwd_kernel(
 // NV = 16-byte chunks per thread and row (1, 2 or 4, the smallest that covers cols): the column
 // sums cost 3 * NV * V registers, and registers decide how many rows a CU has in flight.  The
 // loads of the next two rows are issued before the current row is reduced.
-template <typename T, int V, int NV, int TPR, int kDrop>
-__global__ __launch_bounds__(256) void bias_dropout_residual_ln_bwd_kernel(
+template <typename T, int V, int NV, int TPR, int kDrop, int kThreads>
+__global__ __launch_bounds__(kThreads, (kThreads == 512 && kDrop != 2) ? 4 : 1)
+void bias_dropout_residual_ln_bwd_kernel(
     const T* __restrict__ dy, const T* __restrict__ z, const float* __restrict__ mean,
     const float* __restrict__ rstd, const T* __restrict__ gamma, T* __restrict__ dx,
     T* __restrict__ dres, float* __restrict__ partial, int64_t rows, int cols, DropoutState s) {
-    constexpr int kRows = 256 / TPR;  // rows in flight per block
+    static_assert(TPR == 256 ? kThreads == 256 : (kThreads == 256 || kThreads == 512),
+                  "a block is one wide row, or four or eight wavefront rows");
+    constexpr int kRows = kThreads / TPR;  // rows in flight per block
     constexpr int kIters = kLnRowsPerBlock / kRows;
     constexpr int kCombCols = TPR == 64 ? 64 * V * NV : 1;
     __shared__ float red[2][2][4];
-    __shared__ float comb[kRows * 3 * kCombCols];
+    __shared__ float comb[4 * 3 * kCombCols];
     const int sub = threadIdx.x % TPR;
     const int rr = threadIdx.x / TPR;
     Chunk<T, V> gm[NV];
@@ -559,21 +562,57 @@ __global__ __launch_bounds__(256) void bias_dropout_residual_ln_bwd_kernel(
         // every wavefront (row group) parks its sums in LDS, then the block adds the four copies
         // column by column and writes the partial row with consecutive lanes on consecutive
         // columns
-        float* mine = comb + rr * 3 * kCombCols;
+        float* mine = comb + (rr & 3) * 3 * kCombCols;
+        if constexpr (kRows == 8) {
+            // the upper four wavefronts hand their sums to the lower four first, so that the
+            // parking area stays at four copies
+            if (rr >= 4) {
 #pragma unroll
-        for (int u = 0; u < NV; ++u) {
-            const int col0 = (sub + u * TPR) * V;
-            if (col0 < cols) {
+                for (int u = 0; u < NV; ++u) {
+                    const int col0 = (sub + u * TPR) * V;
+                    if (col0 < cols) {
 #pragma unroll
-                for (int i = 0; i < V; ++i) {
-                    mine[col0 + i] = acc_g[u][i];
-                    mine[kCombCols + col0 + i] = acc_b[u][i];
-                    mine[2 * kCombCols + col0 + i] = acc_x[u][i];
+                        for (int i = 0; i < V; ++i) {
+                            mine[col0 + i] = acc_g[u][i];
+                            mine[kCombCols + col0 + i] = acc_b[u][i];
+                            mine[2 * kCombCols + col0 + i] = acc_x[u][i];
+                        }
+                    }
+                }
+            }
+            __syncthreads();
+            if (rr < 4) {
+#pragma unroll
+                for (int u = 0; u < NV; ++u) {
+                    const int col0 = (sub + u * TPR) * V;
+                    if (col0 < cols) {
+#pragma unroll
+                        for (int i = 0; i < V; ++i) {
+                            acc_g[u][i] += mine[col0 + i];
+                            acc_b[u][i] += mine[kCombCols + col0 + i];
+                            acc_x[u][i] += mine[2 * kCombCols + col0 + i];
+                        }
+                    }
+                }
+            }
+            __syncthreads();
+        }
+        if (rr < 4) {
+#pragma unroll
+            for (int u = 0; u < NV; ++u) {
+                const int col0 = (sub + u * TPR) * V;
+                if (col0 < cols) {
+#pragma unroll
+                    for (int i = 0; i < V; ++i) {
+                        mine[col0 + i] = acc_g[u][i];
+                        mine[kCombCols + col0 + i] = acc_b[u][i];
+                        mine[2 * kCombCols + col0 + i] = acc_x[u][i];
+                    }
                 }
             }
         }
         __syncthreads();
-        for (int c = threadIdx.x; c < 3 * cols; c += 256) {
+        for (int c = threadIdx.x; c < 3 * cols; c += kThreads) {
             const int which = c / cols;
             const int idx = which * kCombCols + (c - which * cols);
             out[c] = (comb[idx] + comb[3 * kCombCols + idx]) +
@@ -842,10 +881,10 @@ int ln_bwd_dispatch(const void* dy, const void* z, const float* mean, const floa
     float* partial = want_sums ? (float*)ws : nullptr;
     const int mode = !dropout ? 0 : (s.g_shift >= 0 && s.t_shift >= 0) ? 1 : 2;
 #define SLAPO_LAUNCH_LNB(NV, TPR, MODE)                                                         \
-    hipLaunchKernelGGL((bias_dropout_residual_ln_bwd_kernel<T, V, NV, TPR, MODE>),              \
-                       dim3((unsigned)n_blocks), dim3(256), 0, st, (const T*)dy, (const T*)z,   \
-                       mean, rstd, (const T*)gamma, (T*)dx, (T*)dres, partial, rows, (int)cols, \
-                       s)
+    hipLaunchKernelGGL(                                                                         \
+        (bias_dropout_residual_ln_bwd_kernel<T, V, NV, TPR, MODE, (TPR == 64 ? 512 : 256)>),    \
+        dim3((unsigned)n_blocks), dim3(TPR == 64 ? 512 : 256), 0, st, (const T*)dy,             \
+        (const T*)z, mean, rstd, (const T*)gamma, (T*)dx, (T*)dres, partial, rows, (int)cols, s)
 #define SLAPO_LAUNCH_LNB_MODE(NV, TPR)            \
     do {                                          \
         if (mode == 0) SLAPO_LAUNCH_LNB(NV, TPR, 0); \
