@@ -13,6 +13,8 @@ roofline  the dK/dV backward kernel (the dominant kernel): its algorithmic FLOPs
           dense fp16 MFMA peak; "kernels" lists the same figure for the forward and dQ kernels
 epilogue  GB/s of the two FusedMLP epilogues (bf16, tokens 8192, 1024 -> 4096 -> 1024) against the
           HBM peak, on a rotating working set larger than the caches
+other_attention  forward and backward time of the OPT-2.7B-shaped (padding mask) and the two
+          GPT-Neo-1.3B-shaped (global / window 256, dropout 0.1) attention calls, bf16
 cpu_baseline  the oracle's native-PyTorch restatement (fp32 CPU, autograd backward) timed on the
           host cores on a bounded sample of the same workload
 """
@@ -272,6 +274,91 @@ def cpu_baseline(cfg, budget_batches=8):
                       f"(fp32 math on fp16 inputs, median of 3, {sec:.2f} s per pass)"}
 
 
+OTHER_ATTENTION = [
+    dict(name="opt-2.7b causal + key-padding attention fwd+bwd", batch=4, seq=2048, heads=32,
+         head_dim=80, window=0, p=0.0, padding=True),
+    dict(name="gpt-neo-1.3b global causal attention fwd+bwd, dropout 0.1", batch=4, seq=2048,
+         heads=16, head_dim=128, window=0, p=0.1, padding=False),
+    dict(name="gpt-neo-1.3b local causal attention (window 256) fwd+bwd, dropout 0.1", batch=4,
+         seq=2048, heads=16, head_dim=128, window=256, p=0.1, padding=False),
+]
+
+
+def bench_other_attention(device, iters=20):
+    """Forward and backward time of the other attention shapes of the benchmark set (bf16), through
+    the C ABI on preallocated buffers; TFLOP/s count 14 * D FLOP per attended (query, key) pair.
+    The padding mask is the compact additive [B,1,1,Sk] tensor with per-sequence valid lengths
+    ~ Uniform[512, 2048]; with dropout the backward reads the keep bits the forward stored."""
+    from slapo_amd import _lib
+    from slapo_amd.op import _kernels as K
+
+    lib = _lib.load()
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    P = lambda t: ctypes.c_void_p(t.data_ptr()) if t is not None else None
+    bf = torch.bfloat16
+    out = []
+    for cfg in OTHER_ATTENTION:
+        B, S, H, D = cfg["batch"], cfg["seq"], cfg["heads"], cfg["head_dim"]
+        g = torch.Generator().manual_seed(2013)
+        q, k, v, do = (torch.randn((B, S, H, D), generator=g).to(bf).to(device) for _ in range(4))
+        bias, lens = None, [S] * B
+        if cfg["padding"]:
+            lens = torch.randint(512, S + 1, (B,), generator=g).tolist()
+            m = torch.zeros(B, 1, 1, S)
+            for i, n in enumerate(lens):
+                m[i, 0, 0, n:] = torch.finfo(bf).min
+            bias = K.prepare_bias(m.to(device), B, H, S, S)
+        w = cfg["window"]
+        pairs = 0
+        for n in lens:  # query i sees keys max(0, i - w + 1) .. min(i, n - 1)
+            for i in range(S):
+                lo = max(0, i - w + 1) if w else 0
+                pairs += max(0, min(i, n - 1) - lo + 1)
+        pairs *= H
+        plan = K.dropout_plan(B * H * S * S, 4, q.device) if cfg["p"] > 0 else None
+        scale = D ** -0.5
+        o, lse, _, keep = K.attn_fwd(q, k, v, bias, True, w, scale, cfg["p"], 2013, 0, plan,
+                                     save_mask=True)
+        prm = K.make_attn_params(q, k, v, o, bias, True, w, scale, cfg["p"], 2013, 0, plan, keep)
+        dq, dk, dv = (torch.empty_like(q) for _ in range(3))
+        nbytes = lib.slapo_amd_attn_bwd_workspace_bytes(ctypes.byref(prm))
+        ws = torch.empty(nbytes // 4, dtype=torch.float32, device=device)
+        strides = [K._bshd_strides(t) for t in (dq, dk, dv)]
+
+        def fwd():
+            rc = lib.slapo_amd_attn_fwd(ctypes.byref(prm), P(q), P(k), P(v), P(bias), P(o), P(lse),
+                                        st)
+            if rc:
+                raise RuntimeError(f"slapo_amd_attn_fwd failed with status {rc}")
+
+        def bwd():
+            rc = lib.slapo_amd_attn_bwd(ctypes.byref(prm), P(q), P(k), P(v), P(bias), P(o), P(do),
+                                        P(lse), P(dq), P(dk), P(dv), *strides, P(ws), nbytes, st)
+            if rc:
+                raise RuntimeError(f"slapo_amd_attn_bwd failed with status {rc}")
+
+        def timed(fn):
+            for _ in range(3):
+                fn()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            for _ in range(iters):
+                fn()
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) / iters * 1e-3
+
+        tf, tb = timed(fwd), timed(bwd)
+        tflops = 14 * D * pairs / (tf + tb) / 1e12
+        out.append({"workload": cfg["name"], "dtype": "bf16", "batch": B, "seq_len": S, "heads": H,
+                    "head_dim": D, "window": w, "dropout_p": cfg["p"], "attended_pairs": pairs,
+                    "fwd_us": tf * 1e6, "bwd_us": tb * 1e6, "TFLOPs": tflops,
+                    "frac_of_mfma_peak": tflops / MFMA_PEAK_TFLOPS})
+        del q, k, v, do, o, lse, dq, dk, dv, ws, keep, bias
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -279,6 +366,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-epilogues", action="store_true")
+    ap.add_argument("--no-other-attention", action="store_true",
+                    help="skip the other attention shapes of the benchmark set")
     ap.add_argument("--traffic-reference", action="store_true",
                     help="also run three 256 MiB device-to-device copies, the known-size kernel "
                          "against which FETCH_SIZE / WRITE_SIZE counter readings are scaled")
@@ -358,6 +447,8 @@ def main():
                          kern("attn_bwd_dq_kernel<f16, 64, false, 0, true>", 6 * d * n_pairs, seg_ms[1])]
     if not args.no_epilogues:
         result["epilogue"] = bench_epilogues(device)
+    if not args.no_other_attention:
+        result["other_attention"] = bench_other_attention(device)
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(cfg)
     print(json.dumps(result))
