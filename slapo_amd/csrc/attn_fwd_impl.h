@@ -32,15 +32,16 @@ constexpr int kBM = kWaves * 32;
 constexpr int kBN = 64;
 constexpr float kMaxSlack = 8.0f;  // hysteresis of the softmax reference, log2 units
 
-template <typename T, int DPAD, bool kBias, int kDrop, bool kWin>
+template <typename T, int DPAD, bool kBias, int kDrop, int kWin>
 __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void attn_fwd_kernel(
     const AttnArgs a_in) {
-    // kWin == false: the launcher guarantees window <= 0; folding that in removes the two-sided
-    // mask body and the window tests from the kernel, and with them the register spills of the
-    // bias-free builds (head_dim 64: 24 spilled registers -> none, 37.8 -> 35.7 us at fp16 B8
-    // S1024 H16 causal; head_dim 128: 69 -> 4, 116 -> 96-109 us at bf16 B4 S2048 H16 causal)
+    // kWin: 0 = the launcher guarantees window <= 0, 1 = it guarantees window > 0, 2 = either.
+    // Folding "no window" in removes the two-sided mask body and the window tests from the
+    // kernel, and with them the register spills of the bias-free builds (head_dim 64: 24 spilled
+    // registers -> none, 37.8 -> 35.7 us at fp16 B8 S1024 H16 causal; head_dim 128: 69 -> 4,
+    // 116 -> 96-109 us at bf16 B4 S2048 H16 causal); folding "window" in leaves one masked body.
     AttnArgs a = a_in;
-    if constexpr (!kWin) a.window = 0;
+    if constexpr (kWin == 0) a.window = 0;
     typedef typename Mma<T>::frag frag_t;
     typedef TileStage<T, DPAD, kBN, kThreads> Stage;
     constexpr int kPitch = Stage::kPitch;
@@ -327,7 +328,9 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
             if (tile_active(t)) {
                 if (!tile_needs_mask(t))
                     tile_body(kt, vt, t, std::integral_constant<int, 0>{});
-                else if (kWin && a.window > 0)
+                else if constexpr (kWin == 1)  // one masked body per build: both bounds
+                    tile_body(kt, vt, t, std::integral_constant<int, 2>{});
+                else if (kWin == 2 && a.window > 0)
                     tile_body(kt, vt, t, std::integral_constant<int, 2>{});
                 else
                     tile_body(kt, vt, t, std::integral_constant<int, 1>{});
@@ -341,16 +344,35 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
         }
         __syncthreads();
     };
-    // leading tiles that need neither mask nor activity test for any of the 128 queries
-    int n_fast = 0;
-    if (a.window <= 0 && q0 + kBM <= a.sq) {
-        n_fast = a.sk / kBN;
-        if (a.causal) n_fast = min(n_fast, (q0 + 1) / kBN);
-        n_fast = min(n_fast, n_tiles);
+    // tiles that need neither mask nor activity test for any of the 128 queries: the leading
+    // ones without a local window, a run in the middle of the key range with one
+    if constexpr (kWin != 1) {
+        int n_fast = 0;
+        if (a.window <= 0 && q0 + kBM <= a.sq) {
+            n_fast = a.sk / kBN;
+            if (a.causal) n_fast = min(n_fast, (q0 + 1) / kBN);
+            n_fast = min(n_fast, n_tiles);
+        }
+        int r = 0;
+        for (; r < n_fast; ++r) iteration(r, std::true_type{});
+        for (; r < n_tiles; ++r) iteration(r, std::false_type{});
+    } else {
+        int f_lo = 0, f_hi = 0;  // iterations [f_lo, f_hi) are fast
+        if (q0 + kBM <= a.sq) {
+            int t_end = a.sk / kBN;  // first tile that is incomplete or hidden from some query
+            if (a.causal) t_end = min(t_end, (q0 + 1) / kBN);
+            // the last query of the workgroup sees keys >= q0 + kBM - window
+            const int t_begin = (max(q0 + kBM - a.window, 0) + kBN - 1) / kBN;
+            f_lo = min(max(t_begin - t_lo, 0), n_tiles);
+            f_hi = min(max(t_end - t_lo, f_lo), n_tiles);
+        }
+        for (int r = 0; r < n_tiles; ++r) {
+            if (r >= f_lo && r < f_hi)
+                iteration(r, std::true_type{});
+            else
+                iteration(r, std::false_type{});
+        }
     }
-    int r = 0;
-    for (; r < n_fast; ++r) iteration(r, std::true_type{});
-    for (; r < n_tiles; ++r) iteration(r, std::false_type{});
 
     // ---- epilogue ----
     const float l_tot = sum_xor32(l_run);
@@ -376,7 +398,7 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
     }
 }
 
-template <typename T, int DPAD, bool kBias, int kDrop, bool kWin>
+template <typename T, int DPAD, bool kBias, int kDrop, int kWin>
 int launch(const AttnArgs& a, hipStream_t st) {
     typedef TileStage<T, DPAD, kBN, kThreads> Stage;
     const size_t smem = (size_t)4 * kBN * Stage::kPitch * sizeof(T);
@@ -398,7 +420,7 @@ int launch(const AttnArgs& a, hipStream_t st) {
     return check_launch();
 }
 
-template <typename T, int DPAD, bool kWin>
+template <typename T, int DPAD, int kWin>
 int dispatch_nobias(const AttnArgs& a, hipStream_t st) {
     if (a.dropout == 1) return launch<T, DPAD, false, 1, kWin>(a, st);
     if (a.dropout == 2) return launch<T, DPAD, false, 2, kWin>(a, st);
@@ -409,12 +431,11 @@ int dispatch_flags(const AttnArgs& a, hipStream_t st) {
     if (a.has_bias) {
         // one build for both: with a bias the window-free build measured slower (it spills more
         // at head_dim 64 and 96: 266 against 185 us at bf16 B4 S2048 H32 D80 with a padding mask)
-        if (a.dropout == 1) return launch<T, DPAD, true, 1, true>(a, st);
-        if (a.dropout == 2) return launch<T, DPAD, true, 2, true>(a, st);
-        return launch<T, DPAD, true, 0, true>(a, st);
+        if (a.dropout == 1) return launch<T, DPAD, true, 1, 2>(a, st);
+        if (a.dropout == 2) return launch<T, DPAD, true, 2, 2>(a, st);
+        return launch<T, DPAD, true, 0, 2>(a, st);
     }
-    return a.window > 0 ? dispatch_nobias<T, DPAD, true>(a, st)
-                        : dispatch_nobias<T, DPAD, false>(a, st);
+    return a.window > 0 ? dispatch_nobias<T, DPAD, 1>(a, st) : dispatch_nobias<T, DPAD, 0>(a, st);
 }
 
 template <typename T>
