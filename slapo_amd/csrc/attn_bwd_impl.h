@@ -229,8 +229,10 @@ __global__ __launch_bounds__(kBwdThreads, (bwd_two_per_cu(DPAD, kDrop, KB) ? 2 :
     };
     auto tile_fast = [&](int t) __attribute__((always_inline)) {
         const int i0 = t * kBwdBM;
-        return a.window <= 0 && k0 + kBN <= a.sk && i0 + kBwdBM <= a.sq &&
-               (!a.causal || i0 >= k0 + kBN - 1);
+        // every (query, key) pair of the tile is visible: the first query sees the last key
+        // (causal), the last query still sees the first key (local window)
+        return k0 + kBN <= a.sk && i0 + kBwdBM <= a.sq && (!a.causal || i0 >= k0 + kBN - 1) &&
+               (a.window <= 0 || i0 + kBwdBM - 1 - k0 < a.window);
     };
     // Two generic (diagonal / tail) tiles in a row are processed together, see generic_step; when
     // the kernel starts with such a pair, both tiles are requested at once.
