@@ -190,7 +190,14 @@ __global__ __launch_bounds__(kBwdThreads, (bwd_two_per_cu(DPAD, kDrop, KB) ? 2 :
         const int i0 = t * kBwdBM;
         r.q.load(q_base, a.qs[1], i0, a.sq, a.d);
         r.g.load(g_base, a.os[1], i0, a.sq, a.d);
-        if (threadIdx.x < 2 * kBwdBM)
+        // every thread loads (the upper half of the workgroup a duplicate that stage_tile drops):
+        // a branch here would end the basic block in the middle of a tile body, and the
+        // exponentials of the body then sink below it, away from the matrix instructions that
+        // are meant to run beside them (bf16 B4 S2048 H32 D80 causal: 289 -> 263 us; head_dim 128
+        // with dropout: 236 -> 221 us; head_dim 64: 1-3 %).  Only head_dim 128 without dropout,
+        // which requests at the top of the body, measured better with the branch (659 against
+        // 697 us at S 4096) and keeps it.
+        if (!(DPAD > 96 && kDrop == 0) || threadIdx.x < 2 * kBwdBM)
             r.stat = stat_src[min(i0 + (int)(threadIdx.x & (kBwdBM - 1)), a.sq - 1)];
         if constexpr (kDrop == 3) {
             // the keep bits that the forward stored: thread (w, row) of the workgroup fetches the
