@@ -139,6 +139,17 @@ def test_local_window(dtype, window):
     _check(q, k, v, do, None, True, window, dtype)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(1, 700, 2, 64), (1, 640, 1, 128), (2, 520, 1, 80)])
+@pytest.mark.parametrize("window", [130, 192, 256, 333])
+def test_local_window_with_mask_free_tiles_inside(dtype, shape, window):
+    """Windows wide enough that whole key tiles (forward) and query tiles (dK/dV) lie inside the
+    window for every row of a workgroup: those tiles take the mask-free path between the masked
+    tiles of the window's lower edge and of the diagonal; ragged last tiles as well."""
+    q, k, v, do, _ = _inputs(*shape, dtype)
+    _check(q, k, v, do, None, True, window, dtype)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float16])
 @pytest.mark.parametrize("sq,sk", [(64, 192), (130, 70), (1, 257)])
 def test_cross_lengths(dtype, sq, sk):
