@@ -32,9 +32,14 @@ constexpr int kBM = kWaves * 32;
 constexpr int kBN = 64;
 constexpr float kMaxSlack = 8.0f;  // hysteresis of the softmax reference, log2 units
 
-template <typename T, int DPAD, bool kBias, int kDrop, int kWin>
+template <typename T, int DPAD, int kBias, int kDrop, int kWin>
 __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void attn_fwd_kernel(
     const AttnArgs a_in) {
+    // kBias: 0 = no additive bias, 1 = any layout (read from memory per score), 2 = the bias
+    // depends on the key only (stride 0 over the queries, e.g. a [B,1,1,Sk] padding mask): the 64
+    // values of a key tile travel through LDS beside the K / V tile and the tile body has neither
+    // global loads nor branches for them (bf16 B4 S2048 H32 D80 causal, every key valid: 241 us
+    // with the per-score reads against 169 us without a bias).
     // kWin: 0 = the launcher guarantees window <= 0, 1 = it guarantees window > 0, 2 = either.
     // Folding "no window" in removes the two-sided mask body and the window tests from the
     // kernel, and with them the register spills of the bias-free builds (head_dim 64: 24 spilled
@@ -52,6 +57,7 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
     extern __shared__ __align__(16) unsigned char smem_raw[];
     T* k_lds = reinterpret_cast<T*>(smem_raw);  // K[2][tile]
     T* v_lds = k_lds + 2 * kTileElems;          // V[2][tile]
+    float* bias_lds = reinterpret_cast<float*>(v_lds + 2 * kTileElems);  // [2][kBN], kBias == 2
 
     const int n_bh = a.batch * a.heads;
     const int n_qt = (a.sq + kBM - 1) / kBM;
@@ -122,6 +128,20 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
     const float* bias_row = nullptr;
     if constexpr (kBias)
         bias_row = a.bias + b * a.bs[0] + h * a.bs[1] + (int64_t)min(q_row, a.sq - 1) * a.bs[2];
+    // kBias == 2: thread (x & 63) carries key j0 + (x & 63) of the requested tile (all four
+    // wavefronts alike, so that neither request nor store needs a branch)
+    const float* bias_keys = nullptr;
+    if constexpr (kBias == 2) bias_keys = a.bias + b * a.bs[0] + h * a.bs[1];
+    float bias_stage = 0.f;
+    auto request_bias = [&](int j0) __attribute__((always_inline)) {
+        if constexpr (kBias == 2)
+            bias_stage = bias_keys[(int64_t)min(j0 + lane, a.sk - 1) * a.bs[3]];
+    };
+    auto store_bias = [&](int slot) __attribute__((always_inline)) {
+        if constexpr (kBias == 2) bias_lds[slot * kBN + lane] = bias_stage * kLog2e;
+    };
+    const float* bias_tile = bias_lds;  // the slot of the tile in process
+    request_bias(t_lo * kBN);
 
     // per-lane LDS offsets (elements) that do not change from tile to tile
     const int k_off = pi_row(i_loc) * kPitch + 8 * g;
@@ -165,7 +185,14 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
         float mx = -INFINITY;
 #pragma unroll
         for (int r4 = 0; r4 < 4; ++r4) {
-            if constexpr (kBias) {
+            if constexpr (kBias == 2) {
+                const f32x4_t t4 = *reinterpret_cast<const f32x4_t*>(bias_tile + 32 * kb +
+                                                                     acc_row(4 * r4, g));
+                s[4 * r4 + 0] = __builtin_fmaf(s[4 * r4 + 0], c_log2, t4.x);
+                s[4 * r4 + 1] = __builtin_fmaf(s[4 * r4 + 1], c_log2, t4.y);
+                s[4 * r4 + 2] = __builtin_fmaf(s[4 * r4 + 2], c_log2, t4.z);
+                s[4 * r4 + 3] = __builtin_fmaf(s[4 * r4 + 3], c_log2, t4.w);
+            } else if constexpr (kBias == 1) {
                 const int key0 = j0 + acc_row(4 * r4, g);
                 float bv[4] = {0.f, 0.f, 0.f, 0.f};
                 if (a.bias_vec4 && key0 + 3 < a.sk) {
@@ -307,6 +334,7 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
     vs.fix(t_lo * kBN, a.sk, a.d);
     ks.store(k_lds);
     vs.store(v_lds);
+    store_bias(0);
     __syncthreads();
 
     // Iteration r: request tile r+1, process tile r, write tile r+1 into the other slot.
@@ -320,8 +348,10 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
         // later in the body saves no registers and measures slower.
         ks.load_indexed(k_base, a.ks[1], (t + 1) * kBN, a.sk, a.d);
         vs.load_indexed(v_base, a.vs[1], (t + 1) * kBN, a.sk, a.d);
+        request_bias((t + 1) * kBN);
         const T* kt = k_lds + (r & 1) * kTileElems;
         const T* vt = v_lds + (r & 1) * kTileElems;
+        bias_tile = bias_lds + (r & 1) * kBN;
         if constexpr (kFast) {
             tile_body(kt, vt, t, std::integral_constant<int, 0>{});
         } else {
@@ -341,6 +371,7 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
             vs.fix((t + 1) * kBN, a.sk, a.d);
             ks.store(k_lds + ((r + 1) & 1) * kTileElems);
             vs.store(v_lds + ((r + 1) & 1) * kTileElems);
+            store_bias((r + 1) & 1);
         }
         __syncthreads();
     };
@@ -398,10 +429,11 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
     }
 }
 
-template <typename T, int DPAD, bool kBias, int kDrop, int kWin>
+template <typename T, int DPAD, int kBias, int kDrop, int kWin>
 int launch(const AttnArgs& a, hipStream_t st) {
     typedef TileStage<T, DPAD, kBN, kThreads> Stage;
-    const size_t smem = (size_t)4 * kBN * Stage::kPitch * sizeof(T);
+    const size_t smem = (size_t)4 * kBN * Stage::kPitch * sizeof(T) +
+                        (kBias == 2 ? 2 * kBN * sizeof(float) : 0);
     const int n_qt = (a.sq + kBM - 1) / kBM;
     const int64_t blocks = (int64_t)n_qt * a.batch * a.heads;
     if (blocks <= 0 || blocks > 0x7FFFFFFF) return SLAPO_ERR_SHAPE;
@@ -422,18 +454,24 @@ int launch(const AttnArgs& a, hipStream_t st) {
 
 template <typename T, int DPAD, int kWin>
 int dispatch_nobias(const AttnArgs& a, hipStream_t st) {
-    if (a.dropout == 1) return launch<T, DPAD, false, 1, kWin>(a, st);
-    if (a.dropout == 2) return launch<T, DPAD, false, 2, kWin>(a, st);
-    return launch<T, DPAD, false, 0, kWin>(a, st);
+    if (a.dropout == 1) return launch<T, DPAD, 0, 1, kWin>(a, st);
+    if (a.dropout == 2) return launch<T, DPAD, 0, 2, kWin>(a, st);
+    return launch<T, DPAD, 0, 0, kWin>(a, st);
 }
 template <typename T, int DPAD>
 int dispatch_flags(const AttnArgs& a, hipStream_t st) {
     if (a.has_bias) {
         // one build for both: with a bias the window-free build measured slower (it spills more
         // at head_dim 64 and 96: 266 against 185 us at bf16 B4 S2048 H32 D80 with a padding mask)
-        if (a.dropout == 1) return launch<T, DPAD, true, 1, 2>(a, st);
-        if (a.dropout == 2) return launch<T, DPAD, true, 2, 2>(a, st);
-        return launch<T, DPAD, true, 0, 2>(a, st);
+        if (a.bs[2] == 0) {  // the bias depends on the key only
+            if (a.dropout == 1) return launch<T, DPAD, 2, 1, 2>(a, st);
+            if (a.dropout == 2) return launch<T, DPAD, 2, 2, 2>(a, st);
+            if (a.window <= 0) return launch<T, DPAD, 2, 0, 0>(a, st);
+            return launch<T, DPAD, 2, 0, 2>(a, st);
+        }
+        if (a.dropout == 1) return launch<T, DPAD, 1, 1, 2>(a, st);
+        if (a.dropout == 2) return launch<T, DPAD, 1, 2, 2>(a, st);
+        return launch<T, DPAD, 1, 0, 2>(a, st);
     }
     return a.window > 0 ? dispatch_nobias<T, DPAD, 1>(a, st) : dispatch_nobias<T, DPAD, 0>(a, st);
 }
