@@ -34,7 +34,10 @@ constexpr int kVRing = 2;
 
 // kStagger: see the tile bodies below.  Staggered halves need one workgroup per CU above
 // head_dim 64; sequential halves fit two.
-template <typename T, int DPAD, bool kBias, int kDrop, bool kStagger>
+// kBias: 0 = no additive bias, 1 = any layout (read from memory per score), 2 = the bias depends on
+// the key only (stride 0 over the queries): its 64 values per key tile travel through LDS beside
+// the K / V tile, and the tile bodies have neither global loads nor branches for them.
+template <typename T, int DPAD, int kBias, int kDrop, bool kStagger>
 __global__ __launch_bounds__(kThreads, (kStagger && DPAD > 64 ? 1 : 2)) void attn_bwd_dq_kernel(
     const AttnArgs a) {
     typedef typename Mma<T>::frag frag_t;
@@ -48,6 +51,7 @@ __global__ __launch_bounds__(kThreads, (kStagger && DPAD > 64 ? 1 : 2)) void att
     T* smem = reinterpret_cast<T*>(smem_raw);
     T* k_lds = smem;                        // K[kKRing][tile]
     T* v_lds = smem + kKRing * kTileElems;  // V[kVRing][tile]
+    float* bias_lds = reinterpret_cast<float*>(smem + (kKRing + kVRing) * kTileElems);  // [2][kBN]
 
     const int n_bh = a.batch * a.heads;
     const int n_qt = (a.sq + kBM - 1) / kBM;
@@ -80,7 +84,18 @@ __global__ __launch_bounds__(kThreads, (kStagger && DPAD > 64 ? 1 : 2)) void att
         ks.init(a.ks[1], a.d);
         vs.init(a.vs[1], a.d);
     }
+    // kBias == 2: thread (x & 63) carries key row0 + (x & 63) of the requested tile (all four
+    // wavefronts alike, so that neither request nor store needs a branch)
+    const float* bias_keys = nullptr;
+    if constexpr (kBias == 2) bias_keys = a.bias + b * a.bs[0] + h * a.bs[1];
+    float bias_stage = 0.f;
+    auto store_bias = [&](int slot) __attribute__((always_inline)) {
+        if constexpr (kBias == 2) bias_lds[slot * kBN + lane] = bias_stage * kLog2e;
+    };
+    const float* bias_tile = bias_lds;  // the slot of the tile in process
     auto request = [&](int row0) __attribute__((always_inline)) {
+        if constexpr (kBias == 2)
+            bias_stage = bias_keys[(int64_t)min(row0 + lane, a.sk - 1) * a.bs[3]];
         if constexpr (kIndexed) {
             ks.load_indexed(k_base, a.ks[1], row0, a.sk, a.d);
             vs.load_indexed(v_base, a.vs[1], row0, a.sk, a.d);
@@ -238,7 +253,11 @@ __global__ __launch_bounds__(kThreads, (kStagger && DPAD > 64 ? 1 : 2)) void att
 #pragma unroll
         for (int r4 = 0; r4 < 4; ++r4) {
             float bv[4] = {0.f, 0.f, 0.f, 0.f};
-            if constexpr (kBias) {
+            if constexpr (kBias == 2) {  // already in log2 units
+                const f32x4_t t4 = *reinterpret_cast<const f32x4_t*>(bias_tile + 32 * kb +
+                                                                     acc_row(4 * r4, g));
+                bv[0] = t4.x, bv[1] = t4.y, bv[2] = t4.z, bv[3] = t4.w;
+            } else if constexpr (kBias == 1) {
                 const int key0 = j0 + acc_row(4 * r4, g);
                 if (a.bias_vec4 && key0 + 3 < a.sk) {
                     const f32x4_t t4 = *reinterpret_cast<const f32x4_t*>(bias_row + key0);
@@ -252,7 +271,8 @@ __global__ __launch_bounds__(kThreads, (kStagger && DPAD > 64 ? 1 : 2)) void att
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 float x = __builtin_fmaf(s[4 * r4 + e], c_log2, -lse2);
-                if constexpr (kBias) x = __builtin_fmaf(bv[e], kLog2e, x);
+                if constexpr (kBias == 2) x += bv[e];
+                if constexpr (kBias == 1) x = __builtin_fmaf(bv[e], kLog2e, x);
                 float p = fast_exp2(x);
                 if constexpr (kMask != 0) {
                     const int c = acc_row(4 * r4, 0) + e;
@@ -412,6 +432,7 @@ __global__ __launch_bounds__(kThreads, (kStagger && DPAD > 64 ? 1 : 2)) void att
         vs.fix(t_lo * kBN, a.sk, a.d);
         ks.store(k_lds);
         vs.store(v_lds);
+        store_bias(0);
     }
     __syncthreads();
 
@@ -427,6 +448,7 @@ __global__ __launch_bounds__(kThreads, (kStagger && DPAD > 64 ? 1 : 2)) void att
         }
         const T* kt = k_lds + (r % kKRing) * kTileElems;
         const T* vt = v_lds + (r % kVRing) * kTileElems;
+        bias_tile = bias_lds + (r & 1) * kBN;
         if constexpr (kFast) {
             if constexpr (kStagger)
                 tile_body_fast(kt, vt, t);
@@ -445,6 +467,7 @@ __global__ __launch_bounds__(kThreads, (kStagger && DPAD > 64 ? 1 : 2)) void att
             vs.fix((t + 1) * kBN, a.sk, a.d);
             ks.store(k_lds + ((r + 1) % kKRing) * kTileElems);
             vs.store(v_lds + ((r + 1) % kVRing) * kTileElems);
+            store_bias((r + 1) & 1);
         }
         __syncthreads();
     };
@@ -477,10 +500,11 @@ __global__ __launch_bounds__(kThreads, (kStagger && DPAD > 64 ? 1 : 2)) void att
     }
 }
 
-template <typename T, int DPAD, bool kBias, int kDrop, bool kStagger>
+template <typename T, int DPAD, int kBias, int kDrop, bool kStagger>
 int launch(const AttnArgs& a, hipStream_t st) {
     typedef TileStage<T, DPAD, kBN, kThreads> Stage;
-    const size_t smem = (size_t)(kKRing + kVRing) * kBN * Stage::kPitch * sizeof(T);
+    const size_t smem = (size_t)(kKRing + kVRing) * kBN * Stage::kPitch * sizeof(T) +
+                        (kBias == 2 ? 2 * kBN * sizeof(float) : 0);
     const int n_qt = (a.sq + kBM - 1) / kBM;
     const int64_t blocks = (int64_t)n_qt * a.batch * a.heads;
     if (blocks <= 0 || blocks > 0x7FFFFFFF) return SLAPO_ERR_SHAPE;
@@ -502,15 +526,21 @@ int launch(const AttnArgs& a, hipStream_t st) {
 template <typename T, int DPAD, bool kStagger>
 int dispatch_flags(const AttnArgs& a, hipStream_t st) {
     if (a.has_bias) {
-        if (a.dropout == 1) return launch<T, DPAD, true, 1, kStagger>(a, st);
-        if (a.dropout == 2) return launch<T, DPAD, true, 2, kStagger>(a, st);
-        if (a.dropout == 3) return launch<T, DPAD, true, 3, kStagger>(a, st);
-        return launch<T, DPAD, true, 0, kStagger>(a, st);
+        if (a.bs[2] == 0) {  // the bias depends on the key only
+            if (a.dropout == 1) return launch<T, DPAD, 2, 1, kStagger>(a, st);
+            if (a.dropout == 2) return launch<T, DPAD, 2, 2, kStagger>(a, st);
+            if (a.dropout == 3) return launch<T, DPAD, 2, 3, kStagger>(a, st);
+            return launch<T, DPAD, 2, 0, kStagger>(a, st);
+        }
+        if (a.dropout == 1) return launch<T, DPAD, 1, 1, kStagger>(a, st);
+        if (a.dropout == 2) return launch<T, DPAD, 1, 2, kStagger>(a, st);
+        if (a.dropout == 3) return launch<T, DPAD, 1, 3, kStagger>(a, st);
+        return launch<T, DPAD, 1, 0, kStagger>(a, st);
     }
-    if (a.dropout == 1) return launch<T, DPAD, false, 1, kStagger>(a, st);
-    if (a.dropout == 2) return launch<T, DPAD, false, 2, kStagger>(a, st);
-    if (a.dropout == 3) return launch<T, DPAD, false, 3, kStagger>(a, st);
-    return launch<T, DPAD, false, 0, kStagger>(a, st);
+    if (a.dropout == 1) return launch<T, DPAD, 0, 1, kStagger>(a, st);
+    if (a.dropout == 2) return launch<T, DPAD, 0, 2, kStagger>(a, st);
+    if (a.dropout == 3) return launch<T, DPAD, 0, 3, kStagger>(a, st);
+    return launch<T, DPAD, 0, 0, kStagger>(a, st);
 }
 
 template <typename T>
