@@ -51,7 +51,7 @@ constexpr bool bwd_two_per_cu(int dpad, int drop, int kb) {
 // KB = blocks of 32 keys per wavefront.  KB = 2 halves the LDS operand traffic per matrix
 // instruction (every Q / dO fragment read feeds two MFMAs) at the price of twice the resident
 // fragments and accumulators, i.e. one wavefront per SIMD instead of two.
-template <typename T, int DPAD, bool kBias, int kDrop, int KB>
+template <typename T, int DPAD, int kBias, int kDrop, int KB>
 // Two workgroups per CU up to DPAD 96, one at 128 (192 resident accumulator / fragment registers)
 // and at 96 with the forward's keep bits (measured 23-35 % slower with two than with one).
 __global__ __launch_bounds__(kBwdThreads, (bwd_two_per_cu(DPAD, kDrop, KB) ? 2 : 1)) void attn_bwd_kernel(
@@ -128,8 +128,10 @@ __global__ __launch_bounds__(kBwdThreads, (bwd_two_per_cu(DPAD, kDrop, KB) ? 2 :
     const int t_lo = i_lo / kBwdBM;
     const int t_hi = (i_hi + kBwdBM - 1) / kBwdBM;
 
-    // Per-lane bias when it does not depend on the query (the compact [B,1,1,Sk] layout).
-    const bool bias_per_key = kBias && a.bs[2] == 0;
+    // kBias: 0 = none, 1 = any layout (read from memory per score), 2 = the launcher guarantees a
+    // bias that does not depend on the query (stride 0 over the queries, the compact [B,1,1,Sk]
+    // layout): one register per lane and key block.
+    constexpr bool bias_per_key = kBias == 2;
     float bias_k[KB];
 #pragma unroll
     for (int kb = 0; kb < KB; ++kb) {
@@ -341,11 +343,11 @@ __global__ __launch_bounds__(kBwdThreads, (bwd_two_per_cu(DPAD, kDrop, KB) ? 2 :
                         x = s[kb][4 * r4 + e] * c_log2;  // lse already subtracted
                     else
                         x = __builtin_fmaf(s[kb][4 * r4 + e], c_log2, -lse4[e]);
-                    if constexpr (kBias) {
+                    if constexpr (kBias == 2) {
+                        x += bias_k[kb];
+                    } else if constexpr (kBias == 1) {
                         const int i = ih0 + qoff + e;
-                        if (bias_per_key)
-                            x += bias_k[kb];
-                        else if (i < a.sq && key[kb] < a.sk)
+                        if (i < a.sq && key[kb] < a.sk)
                             x += a.bias[b * a.bs[0] + h * a.bs[1] + (int64_t)i * a.bs[2] +
                                         (int64_t)key[kb] * a.bs[3]] * kLog2e;
                     }
@@ -636,7 +638,7 @@ __global__ __launch_bounds__(kBwdThreads, (bwd_two_per_cu(DPAD, kDrop, KB) ? 2 :
     }
 }
 
-template <typename T, int DPAD, bool kBias, int kDrop, int KB>
+template <typename T, int DPAD, int kBias, int kDrop, int KB>
 int launch(const AttnArgs& a, hipStream_t st) {
     typedef BwdSmem<T, DPAD> SM;
     const size_t smem = SM::kBytes;
@@ -662,23 +664,23 @@ int launch(const AttnArgs& a, hipStream_t st) {
 // Two key blocks per wavefront (KB = 2, one wavefront per SIMD) measured slower than KB = 1 with two
 // wavefronts per SIMD on MI355X (92 us against 70 us at fp16 B8 S1024 H16 D64 causal): the second
 // resident wavefront hides more latency than the halved LDS traffic saves.  Only KB = 1 is built.
-template <typename T, int DPAD, bool kBias, int kDrop>
+template <typename T, int DPAD, int kBias, int kDrop>
 int launch_kb(const AttnArgs& a, hipStream_t st) {
     return launch<T, DPAD, kBias, kDrop, 1>(a, st);
 }
 
+template <typename T, int DPAD, int kBias>
+int dispatch_drop(const AttnArgs& a, hipStream_t st) {
+    if (a.dropout == 1) return launch_kb<T, DPAD, kBias, 1>(a, st);
+    if (a.dropout == 2) return launch_kb<T, DPAD, kBias, 2>(a, st);
+    if (a.dropout == 3) return launch_kb<T, DPAD, kBias, 3>(a, st);
+    return launch_kb<T, DPAD, kBias, 0>(a, st);
+}
+
 template <typename T, int DPAD>
 int dispatch_flags(const AttnArgs& a, hipStream_t st) {
-    if (a.has_bias) {
-        if (a.dropout == 1) return launch_kb<T, DPAD, true, 1>(a, st);
-        if (a.dropout == 2) return launch_kb<T, DPAD, true, 2>(a, st);
-        if (a.dropout == 3) return launch_kb<T, DPAD, true, 3>(a, st);
-        return launch_kb<T, DPAD, true, 0>(a, st);
-    }
-    if (a.dropout == 1) return launch_kb<T, DPAD, false, 1>(a, st);
-    if (a.dropout == 2) return launch_kb<T, DPAD, false, 2>(a, st);
-    if (a.dropout == 3) return launch_kb<T, DPAD, false, 3>(a, st);
-    return launch_kb<T, DPAD, false, 0>(a, st);
+    if (!a.has_bias) return dispatch_drop<T, DPAD, 0>(a, st);
+    return a.bs[2] == 0 ? dispatch_drop<T, DPAD, 2>(a, st) : dispatch_drop<T, DPAD, 1>(a, st);
 }
 
 template <typename T>
