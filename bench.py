@@ -436,15 +436,15 @@ def main():
                    "heads": cfg["heads"], "head_dim": cfg["head_dim"], "causal": cfg["causal"],
                    "dropout_p": cfg["p"], "flops_per_step": 14 * d * n_pairs},
         "frac_of_mfma_peak": value / MFMA_PEAK_TFLOPS,
-        "roofline": {"bound": "mfma", "kernel": "attn_bwd_kernel<f16, 64, false, 0> (dK/dV)",
+        "roofline": {"bound": "mfma", "kernel": "attn_bwd_kernel<f16,64,0,0,1> (dK/dV)",
                      "achieved": achieved,
                      "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / MFMA_PEAK_TFLOPS, "traffic": DKDV_TRAFFIC_BYTES,
                      "flops_per_launch": bwd_flops, "avg_launch_ms": kern_ms},
     }
-    result["kernels"] = [kern("attn_fwd_kernel<f16, 64, false, 0>", 4 * d * n_pairs, seg_ms[0]),
-                         kern("attn_bwd_kernel<f16, 64, false, 0> (dK/dV)", bwd_flops, seg_ms[2]),
-                         kern("attn_bwd_dq_kernel<f16, 64, false, 0, true>", 6 * d * n_pairs, seg_ms[1])]
+    result["kernels"] = [kern("attn_fwd_kernel<f16,64,0,0,0>", 4 * d * n_pairs, seg_ms[0]),
+                         kern("attn_bwd_kernel<f16,64,0,0,1> (dK/dV)", bwd_flops, seg_ms[2]),
+                         kern("attn_bwd_dq_kernel<f16,64,0,0,true>", 6 * d * n_pairs, seg_ms[1])]
     if not args.no_epilogues:
         result["epilogue"] = bench_epilogues(device)
     if not args.no_other_attention:
