@@ -210,7 +210,9 @@ typedef struct slapo_attn_params {
     int64_t v_strides[3];
     int64_t o_strides[3];
     /* additive fp32 bias addressed as bias[b*s0 + h*s1 + i*s2 + j*s3]; stride 0 broadcasts
-     * (the reference's "b11k" layout is {Sk, 0, 0, 1}, "bhqk" is {H*Sq*Sk, Sq*Sk, Sk, 1}) */
+     * (the reference's "b11k" layout is {Sk, 0, 0, 1}, "bhqk" is {H*Sq*Sk, Sq*Sk, Sk, 1}).
+     * With s2 == 0 (the bias depends on the key only) the kernels stage the bias of a key tile
+     * through LDS instead of reading it per score: pass a padding mask in that form. */
     int64_t bias_strides[4];
     /* launch plan of the dropout mask over the dense [batch*heads, seqlen_q, seqlen_k] fp32
      * probability tensor (only read when p_drop > 0) */
