@@ -108,6 +108,23 @@ def test_additive_masks(dtype, layout):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape,sk,causal,window,p", [
+    ((2, 150, 3, 64), 150, True, 0, 0.0),     # ragged last key tile
+    ((1, 70, 2, 80), 201, False, 0, 0.0),     # cross lengths, head_dim 80 (padded to 96)
+    ((1, 260, 2, 128), 260, True, 100, 0.0),  # local window, head_dim 128
+    ((2, 130, 2, 64), 130, True, 0, 0.2),     # dropout
+    ((1, 33, 1, 64), 5, False, 0, 0.0),       # fewer keys than one tile
+])
+def test_key_only_bias_per_batch_and_head(dtype, shape, sk, causal, window, p):
+    """A bias of arbitrary values that depends on batch, head and key but not on the query
+    ([B,H,1,Sk], stride 0 over the queries): the layout that the kernels stage through LDS."""
+    b, s, h, d = shape
+    q, k, v, do, g = _inputs(b, s, h, d, dtype, sk=sk)
+    mask = torch.randn(b, h, 1, sk, generator=g).to(dtype)
+    _check(q, k, v, do, mask, causal, window, dtype, p)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("kind", ["short", "left", "holes"])
 def test_padding_masks_and_tile_skipping(dtype, causal, kind):
