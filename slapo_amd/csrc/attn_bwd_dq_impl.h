@@ -11,8 +11,10 @@
 // values stream through LDS in tiles of 64, double buffered and staged through registers (the
 // global loads of tile t+1 are in flight while tile t is processed).  Per key tile, lane l = query
 // i, registers = keys:
-//   S^T  = K Q^T, dP^T = V dO^T    A = K / V rows from LDS (row-permuted 128-bit reads)
-//   P^T  = exp2(S^T * scale - lse), dS^T = P^T * (dP^T - delta)
+//   S^T  = K Q^T, dP^T = V dO^T    A = K / V rows from LDS (row-permuted 128-bit reads); Q carries
+//                                  scale * log2(e), and the accumulators start from -lse and
+//                                  -delta of the lane's query, so that
+//   P^T  = exp2(S^T), dS^T = P^T * dP^T      cost two vector instructions per score
 //   dQ^T += K^T dS^T               B = dS^T straight from the accumulator registers, A = K^T read
 //                                  from the row-major K tile with the transposing LDS read.
 //
@@ -90,7 +92,7 @@ __global__ __launch_bounds__(kThreads, (kStagger && DPAD > 64 ? 1 : 2)) void att
     if constexpr (kBias == 2) bias_keys = a.bias + b * a.bs[0] + h * a.bs[1];
     float bias_stage = 0.f;
     auto store_bias = [&](int slot) __attribute__((always_inline)) {
-        if constexpr (kBias == 2) bias_lds[slot * kBN + lane] = bias_stage * kLog2e;
+        if constexpr (kBias == 2) bias_lds[slot * kBN + row_slot(lane)] = bias_log2(bias_stage);
     };
     const float* bias_tile = bias_lds;  // the slot of the tile in process
     auto request = [&](int row0) __attribute__((always_inline)) {
@@ -135,6 +137,11 @@ __global__ __launch_bounds__(kThreads, (kStagger && DPAD > 64 ? 1 : 2)) void att
             qf[t] = __builtin_bit_cast(frag_t, keep_or_zero(qv[t], keep));
             gf[t] = __builtin_bit_cast(frag_t, keep_or_zero(gv[t], keep));
         }
+        // Q times scale * log2(e), once: the scores leave the matrix pipe in log2 units
+#pragma unroll
+        for (int t = 0; t < DK; ++t) {
+            qf[t] = scale_frag<T>(__builtin_bit_cast(u32x4_t, qf[t]), a.scale_log2);
+        }
         // log2 units; +inf for rows past the end so that P = 0 there
         lse2 = row_ok ? lse_raw * kLog2e : INFINITY;
         // delta = sum_d dO * O: lanes i and i + 32 hold complementary head-dim slots of row i
@@ -149,24 +156,11 @@ __global__ __launch_bounds__(kThreads, (kStagger && DPAD > 64 ? 1 : 2)) void att
         delta = sum_xor32(part);  // masked dO slots are zero, so clamped rows / columns add nothing
         if (row_ok && g == 0) a.delta[(int64_t)bh * a.sq + q_row] = delta;
     }
-    // Without dropout dP^T - delta comes straight out of the matrix pipe: one extra k-step whose A
-    // operand is 1 in k-slots 0..2 (every key row alike) and whose B operand holds -delta of this
-    // lane's query, split into three parts of T whose sum carries at least 24 bits of it, i.e. the
-    // subtraction is as exact as in fp32.
-    frag_t ones_f, ndelta_f;
-    {
-        const float nd = -delta;
-        const T hi = (T)nd;
-        const float r1 = nd - (float)hi;
-        const T mid = (T)r1;
-        const T lo = (T)(r1 - (float)mid);
+    // The per-row terms enter through the accumulators: S^T starts from -lse (log2 units) and,
+    // without dropout, dP^T from -delta, in all sixteen registers of the lane (= one query).
+    f32x16_t neg_lse, neg_delta;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) ones_f[j] = (T)0.f, ndelta_f[j] = (T)0.f;
-        if (g == 0) {
-            ones_f[0] = (T)1.f, ones_f[1] = (T)1.f, ones_f[2] = (T)1.f;
-            ndelta_f[0] = hi, ndelta_f[1] = mid, ndelta_f[2] = lo;
-        }
-    }
+    for (int r = 0; r < 16; ++r) neg_lse[r] = -lse2, neg_delta[r] = kDrop == 0 ? -delta : 0.f;
 
     f32x16_t dq_acc[DV];
 #pragma unroll
@@ -175,7 +169,6 @@ __global__ __launch_bounds__(kThreads, (kStagger && DPAD > 64 ? 1 : 2)) void att
         for (int r = 0; r < 16; ++r) dq_acc[x][r] = 0.f;
 
     const int wq_last = min(wq0 + 31, a.sq - 1);
-    const float c_log2 = a.scale_log2;
     uint64_t drop_row_base = 0;
     if constexpr (kDrop != 0)
         drop_row_base = ((uint64_t)bh * a.sq + (uint64_t)q_row) * (uint64_t)a.sk;
@@ -185,7 +178,7 @@ __global__ __launch_bounds__(kThreads, (kStagger && DPAD > 64 ? 1 : 2)) void att
 
     // per-lane LDS offsets (elements) that do not change from tile to tile
     const int row_off = pi_row(i_loc) * kPitch + 8 * g;
-    const int tr_off = (8 * g + ((lane & 15) >> 2)) * kPitch + ((lane >> 4) & 1) * 16 + 4 * (lane & 3);
+    const int tr_off = tr_lane_off(lane, kPitch);
 
     auto tile_active = [&](int t) __attribute__((always_inline)) {
         if (t < t_lo || t >= t_hi || wq0 >= a.sq) return false;
@@ -208,22 +201,19 @@ __global__ __launch_bounds__(kThreads, (kStagger && DPAD > 64 ? 1 : 2)) void att
     // hides more latency than the stagger does (measured: 28 % faster at head_dim 80, 2-12 % at
     // 128; only the masked tile bodies of a local window lose, to register spills, at 128).
 
-    // S^T half = K_half Q^T
+    // S^T half = K_half Q^T - lse
     auto half_s = [&](const T* kt, int kb, f32x16_t& s) __attribute__((always_inline)) {
+        s = Mma<T>::mma32(lds_frag<T>(kt + kb * 32 * kPitch + row_off), qf[0], neg_lse);
 #pragma unroll
-        for (int r = 0; r < 16; ++r) s[r] = 0.f;
-#pragma unroll
-        for (int x = 0; x < DK; ++x)
+        for (int x = 1; x < DK; ++x)
             s = Mma<T>::mma32(lds_frag<T>(kt + kb * 32 * kPitch + row_off + 16 * x), qf[x], s);
     };
-    // dP^T half = V_half dO^T
+    // dP^T half = V_half dO^T (- delta without dropout)
     auto half_dp = [&](const T* vt, int kb, f32x16_t& dp) __attribute__((always_inline)) {
+        dp = Mma<T>::mma32(lds_frag<T>(vt + kb * 32 * kPitch + row_off), gf[0], neg_delta);
 #pragma unroll
-        for (int r = 0; r < 16; ++r) dp[r] = 0.f;
-#pragma unroll
-        for (int x = 0; x < DK; ++x)
+        for (int x = 1; x < DK; ++x)
             dp = Mma<T>::mma32(lds_frag<T>(vt + kb * 32 * kPitch + row_off + 16 * x), gf[x], dp);
-        if constexpr (kDrop == 0) dp = Mma<T>::mma32(ones_f, ndelta_f, dp);
     };
     // dQ^T += K_half^T dS^T half
     auto half_dq = [&](const T* kt, int kb, const uint32_t (&dw)[8]) __attribute__((always_inline)) {
@@ -243,39 +233,49 @@ __global__ __launch_bounds__(kThreads, (kStagger && DPAD > 64 ? 1 : 2)) void att
     auto half_exp = [&](f32x16_t& s, int t, int kb, auto mask_tag) __attribute__((always_inline)) {
         constexpr int kMask = decltype(mask_tag)::value;
         const int j0 = t * kBN + kb * 32;
-        // register r is key j0 + 8 g + c with c = acc_row(r, 0); visible iff c_lo <= c <= c_hi
+        // register r is key j0 + acc_row(r, g) = j0 + kAccGroupStep g + c with c = acc_row(r, 0);
+        // visible iff c_lo <= c <= c_hi
         int c_lo = 0, c_hi = 0;
         if constexpr (kMask != 0) {
             const int k_max = a.causal ? min(a.sk - 1, q_row) : a.sk - 1;
-            c_hi = k_max - j0 - 8 * g;
-            if constexpr (kMask == 2) c_lo = q_row - a.window + 1 - j0 - 8 * g;
+            c_hi = k_max - j0 - kAccGroupStep * g;
+            if constexpr (kMask == 2) c_lo = q_row - a.window + 1 - j0 - kAccGroupStep * g;
+        }
+        if constexpr (kBias == 1) {
+            // Registers 8 h + e and 8 h + 4 + e are keys 2 g and 2 g + 1 of the aligned group of
+            // four keys at j0 + 16 h + 4 e: one 16-byte read per group where the layout allows.
+#pragma unroll
+            for (int he = 0; he < 8; ++he) {
+                const int kg = j0 + 16 * (he >> 2) + 4 * (he & 3);
+                float b_lo = 0.f, b_hi = 0.f;
+                if (a.bias_vec4 && kg + 3 < a.sk) {
+                    const f32x4_t t4 = *reinterpret_cast<const f32x4_t*>(bias_row + kg);
+                    b_lo = g ? t4.z : t4.x;
+                    b_hi = g ? t4.w : t4.y;
+                } else {
+                    const int k_lo = kg + 2 * g;
+                    if (k_lo < a.sk) b_lo = bias_row[(int64_t)k_lo * a.bs[3]];
+                    if (k_lo + 1 < a.sk) b_hi = bias_row[(int64_t)(k_lo + 1) * a.bs[3]];
+                }
+                s[8 * (he >> 2) + (he & 3)] += bias_log2(b_lo);
+                s[8 * (he >> 2) + 4 + (he & 3)] += bias_log2(b_hi);
+            }
         }
 #pragma unroll
         for (int r4 = 0; r4 < 4; ++r4) {
             float bv[4] = {0.f, 0.f, 0.f, 0.f};
             if constexpr (kBias == 2) {  // already in log2 units
                 const f32x4_t t4 = *reinterpret_cast<const f32x4_t*>(bias_tile + 32 * kb +
-                                                                     acc_row(4 * r4, g));
+                                                                     quad_slot(r4, g));
                 bv[0] = t4.x, bv[1] = t4.y, bv[2] = t4.z, bv[3] = t4.w;
-            } else if constexpr (kBias == 1) {
-                const int key0 = j0 + acc_row(4 * r4, g);
-                if (a.bias_vec4 && key0 + 3 < a.sk) {
-                    const f32x4_t t4 = *reinterpret_cast<const f32x4_t*>(bias_row + key0);
-                    bv[0] = t4.x, bv[1] = t4.y, bv[2] = t4.z, bv[3] = t4.w;
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        if (key0 + e < a.sk) bv[e] = bias_row[(int64_t)(key0 + e) * a.bs[3]];
-                }
             }
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-                float x = __builtin_fmaf(s[4 * r4 + e], c_log2, -lse2);
+                float x = s[4 * r4 + e];  // scale and lse are in already
                 if constexpr (kBias == 2) x += bv[e];
-                if constexpr (kBias == 1) x = __builtin_fmaf(bv[e], kLog2e, x);
                 float p = fast_exp2(x);
                 if constexpr (kMask != 0) {
-                    const int c = acc_row(4 * r4, 0) + e;
+                    const int c = acc_row(4 * r4 + e, 0);
                     if constexpr (kMask == 2) {
                         if (c > c_hi || c < c_lo) p = 0.f;
                     } else {
@@ -300,14 +300,16 @@ __global__ __launch_bounds__(kThreads, (kStagger && DPAD > 64 ? 1 : 2)) void att
     auto half_ds = [&](const f32x16_t& p, const f32x16_t& dp, int t, int kb, uint32_t mword,
                        uint32_t (&dw)[8]) __attribute__((always_inline)) {
         const int j0 = t * kBN + kb * 32;
+        uint32_t word = mword;  // bit j = keep(key j0 + j)
+        if constexpr (kDrop == 1 || kDrop == 2) {
+            // Philox blocks cover four consecutive keys; the two lanes of a query (l, l ^ 32)
+            // draw the blocks of keys 8 g .. 8 g + 7 of each 16-key group and exchange them.
+            word = 0;
 #pragma unroll
-        for (int r4 = 0; r4 < 4; ++r4) {
-            uint32_t bits = 0xFu;
-            if constexpr (kDrop == 3) {
-                bits = (mword >> acc_row(4 * r4, g)) & 0xFu;
-            } else if constexpr (kDrop != 0) {
-                const int key0 = j0 + acc_row(4 * r4, g);
-                bits = 0;
+            for (int blk = 0; blk < 4; ++blk) {
+                const int pos = 16 * (blk >> 1) + 8 * g + 4 * (blk & 1);
+                const int key0 = j0 + pos;
+                uint32_t bits = 0;
                 if (q_row < a.sq && key0 < a.sk) {
                     const uint64_t e0 = drop_row_base + (uint64_t)key0;
                     if constexpr (kDrop == 1)
@@ -315,20 +317,24 @@ __global__ __launch_bounds__(kThreads, (kStagger && DPAD > 64 ? 1 : 2)) void att
                     else
                         bits = dropout_keep_any(a.rng, e0, min(4, a.sk - key0));
                 }
+                word |= bits << pos;
             }
-            float dv[4];
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                float d = dp[4 * r4 + e];
-                if constexpr (kDrop != 0) d = ((bits >> e) & 1u) ? d * a.rng.inv_keep : 0.f;
-                if constexpr (kDrop == 0)
-                    dv[e] = p[4 * r4 + e] * d;  // delta already subtracted by the matrix pipe
-                else
-                    dv[e] = p[4 * r4 + e] * (d - delta);
-            }
-            dw[2 * r4] = pack2<T>(dv[0], dv[1]);
-            dw[2 * r4 + 1] = pack2<T>(dv[2], dv[3]);
+            word = or_xor32(word);
         }
+        const uint32_t word_g = word >> (kAccGroupStep * g);
+        float dv[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            float d = dp[r];
+            if constexpr (kDrop == 0) {
+                dv[r] = p[r] * d;  // delta already subtracted by the matrix pipe
+            } else {
+                d = ((word_g >> acc_row(r, 0)) & 1u) ? d * a.rng.inv_keep : 0.f;
+                dv[r] = p[r] * (d - delta);
+            }
+        }
+#pragma unroll
+        for (int r2 = 0; r2 < 8; ++r2) dw[r2] = pack2<T>(dv[2 * r2], dv[2 * r2 + 1]);
     };
     auto tile_body = [&](const T* kt, const T* vt, int t, auto mask_tag) __attribute__((always_inline)) {
         if constexpr (!kStagger) {
@@ -381,12 +387,11 @@ __global__ __launch_bounds__(kThreads, (kStagger && DPAD > 64 ? 1 : 2)) void att
                     f[s2 * DV + x] =
                         lds_frag_tr<T>(kt + (32 * kb + 16 * s2) * kPitch + tr_off + 32 * x, kPitch);
         };
-        auto mma_rows = [&](const frag_t (&f)[DK], const frag_t (&bfr)[DK], f32x16_t& acc)
-                            __attribute__((always_inline)) {
+        auto mma_rows = [&](const frag_t (&f)[DK], const frag_t (&bfr)[DK], const f32x16_t& init,
+                            f32x16_t& acc) __attribute__((always_inline)) {
+            acc = Mma<T>::mma32(f[0], bfr[0], init);
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[r] = 0.f;
-#pragma unroll
-            for (int x = 0; x < DK; ++x) acc = Mma<T>::mma32(f[x], bfr[x], acc);
+            for (int x = 1; x < DK; ++x) acc = Mma<T>::mma32(f[x], bfr[x], acc);
         };
         auto mma_cols = [&](const frag_t (&f)[2 * DV], const uint32_t (&dw)[8])
                             __attribute__((always_inline)) {
@@ -404,19 +409,17 @@ __global__ __launch_bounds__(kThreads, (kStagger && DPAD > 64 ? 1 : 2)) void att
         rows(vt, 0, vr0);
         __builtin_amdgcn_sched_barrier(0);
         rows(kt, 1, kr1);
-        mma_rows(kr0, qf, s0);
+        mma_rows(kr0, qf, neg_lse, s0);
         __builtin_amdgcn_sched_barrier(0);
         rows(vt, 1, vr1);
-        mma_rows(vr0, gf, p0);
-        if constexpr (kDrop == 0) p0 = Mma<T>::mma32(ones_f, ndelta_f, p0);
+        mma_rows(vr0, gf, neg_delta, p0);
         __builtin_amdgcn_sched_barrier(0);
         cols(0, kq0);
-        mma_rows(kr1, qf, s1);
+        mma_rows(kr1, qf, neg_lse, s1);
         half_exp(s0, t, 0, none);
         __builtin_amdgcn_sched_barrier(0);
         cols(1, kq1);
-        mma_rows(vr1, gf, p1);
-        if constexpr (kDrop == 0) p1 = Mma<T>::mma32(ones_f, ndelta_f, p1);
+        mma_rows(vr1, gf, neg_delta, p1);
         half_ds(s0, p0, t, 0, mw0, dw0);
         __builtin_amdgcn_sched_barrier(0);
         mma_cols(kq0, dw0);
@@ -509,16 +512,9 @@ int launch(const AttnArgs& a, hipStream_t st) {
     const int64_t blocks = (int64_t)n_qt * a.batch * a.heads;
     if (blocks <= 0 || blocks > 0x7FFFFFFF) return SLAPO_ERR_SHAPE;
     auto kern = attn_bwd_dq_kernel<T, DPAD, kBias, kDrop, kStagger>;
-    if (smem > 48 * 1024) {
-        static bool raised = false;  // per instantiation
-        if (!raised) {
-            if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    (int)smem) != hipSuccess)
-                return SLAPO_ERR_LAUNCH;
-            raised = true;
-        }
-    }
+    static std::atomic<uint64_t> lds_ready{0};  // per instantiation, one bit per device
+    if (allow_dynamic_lds(reinterpret_cast<const void*>(kern), smem, lds_ready) != SLAPO_OK)
+        return SLAPO_ERR_LAUNCH;
     hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kThreads), smem, st, a);
     return check_launch();
 }

@@ -6,10 +6,14 @@
 // double buffered and staged through registers.  Per 32-query half tile and wavefront (lane l,
 // g = l / 32):
 //   S  = Q K_w^T, dP = dO V_w^T      A = Q / dO rows from LDS (row-permuted 128-bit reads),
-//                                    B = the resident K_w / V_w fragments.  Lane l holds one KEY
-//                                    column; registers run over 16 query rows.
-//   P  = exp2(S * scale - lse), dS = P * (dP - delta)      recomputed from the saved
-//                                    log-sum-exp; dropout bits regenerated from Philox.
+//                                    B = the resident K_w / V_w fragments (K_w carries scale *
+//                                    log2(e)).  Lane l holds one KEY column; registers run over
+//                                    16 query rows.  The accumulators start from -lse and -delta
+//                                    of their query rows (128-bit LDS reads straight into the
+//                                    accumulator registers), so that
+//   P  = exp2(S), dS = P * dP        cost two vector instructions per score; P is recomputed from
+//                                    the saved log-sum-exp; dropout bits regenerated from Philox
+//                                    or read back from the forward's keep words.
 //   dV_w^T += dO^T P, dK_w^T += Q^T dS    B = P / dS straight from the accumulator registers
 //                                    (the row permutation makes them ordered k-slots), A = dO^T /
 //                                    Q^T read from the same row-major LDS tiles with the
@@ -20,7 +24,6 @@
 // nothing here is shared between workgroups.  One barrier per query tile.
 // Reference semantics: autograd of slapo/op/attention.py:163-181.
 #pragma once
-#include <cstdio>
 #include <type_traits>
 
 #include "attn_common.h"
@@ -139,39 +142,12 @@ __global__ __launch_bounds__(kBwdThreads, (bwd_two_per_cu(DPAD, kDrop, KB) ? 2 :
         if constexpr (kBias) {
             if (bias_per_key && key[kb] < a.sk)
                 bias_k[kb] =
-                    a.bias[b * a.bs[0] + h * a.bs[1] + (int64_t)key[kb] * a.bs[3]] * kLog2e;
+                    bias_log2(a.bias[b * a.bs[0] + h * a.bs[1] + (int64_t)key[kb] * a.bs[3]]);
         }
     }
-    const float c_log2 = a.scale_log2;
-    // Folding the per-row terms into the matrix pipe (below) pays where a workgroup has the CU to
-    // itself (DPAD > 64: 3 % faster); at DPAD 64 it measures the same to 3 % slower.
-    constexpr bool kFold = DPAD > 64;
-    const float inv_scale = 1.0f / a.scale;
-    constexpr float kNoRow = 30000.f;  // fits fp16; scale_log2 * (s - kNoRow) underflows exp2
-
-    // The per-row terms (- lse / scale for S, - delta for dP) are added by the matrix pipe: one
-    // extra k-step whose A operand holds the term of each query row, split into three parts of T
-    // (their sum carries 24 bits) in k-slots 0..2, and whose B operand is 1 in those slots.
-    frag_t ones_f;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) ones_f[j] = (T)0.f;
-    if (g == 0) ones_f[0] = (T)1.f, ones_f[1] = (T)1.f, ones_f[2] = (T)1.f;
-    auto row_term = [&](float v) __attribute__((always_inline)) {
-        const float nv = -v;
-        const T hi = (T)nv;
-        const float r1 = nv - (float)hi;
-        const T mid = (T)r1;
-        const T lo = (T)(r1 - (float)mid);
-        frag_t f;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) f[j] = (T)0.f;
-        if (g == 0) f[0] = hi, f[1] = mid, f[2] = lo;
-        return f;
-    };
-
     // per-lane LDS offsets (elements) that do not change from tile to tile
     const int a_off = pi_row(c_loc) * kPitch + 8 * g;
-    const int t_off = (8 * g + ((lane & 15) >> 2)) * kPitch + ((lane >> 4) & 1) * 16 + 4 * (lane & 3);
+    const int t_off = tr_lane_off(lane, kPitch);
 
     // Registers through which a query tile (Q, dO rows, lse / delta, keep bits) travels from
     // global memory to LDS.
@@ -219,22 +195,16 @@ __global__ __launch_bounds__(kBwdThreads, (bwd_two_per_cu(DPAD, kDrop, KB) ? 2 :
         r.g.store(g_lds + buf * SM::kQTile);
         if (threadIdx.x < 2 * kBwdBM) {
             const bool ok = i0 + (int)(threadIdx.x & (kBwdBM - 1)) < a.sq;
-            // lse in units of the raw dot product (lse / scale), so that exp2(scale_log2 * (s - lse))
-            // is the probability; a large finite value for rows past the end so that P = 0 there;
-            // delta 0
-            // (clamped: a row without any visible key has lse = -inf, and the three-way split
-            // needs finite input)
-            float v;
-            if constexpr (kFold)
-                v = (threadIdx.x < kBwdBM)
-                        ? (ok ? fmaxf(fminf(r.stat * inv_scale, kNoRow), -kNoRow) : kNoRow)
-                        : (ok ? r.stat : 0.f);
-            else  // lse in log2 units, +inf past the end
-                v = (threadIdx.x < kBwdBM) ? (ok ? r.stat * kLog2e : INFINITY)
-                                           : (ok ? r.stat : 0.f);
-            stat_lds[buf * 2 * kBwdBM + threadIdx.x] = v;
+            // what the accumulators start from: -lse in log2 units (-inf past the end, so that
+            // P = 0 there) and, without dropout, -delta; kept at row_slot so that one 128-bit
+            // read returns the values of four accumulator registers in order
+            const float v = (threadIdx.x < kBwdBM)
+                                ? (ok ? -(r.stat * kLog2e) : -INFINITY)
+                                : (ok ? (kDrop == 0 ? -r.stat : r.stat) : 0.f);
+            stat_lds[buf * 2 * kBwdBM + (threadIdx.x & kBwdBM) + row_slot(threadIdx.x & (kBwdBM - 1))] = v;
         }
-        if constexpr (kDrop == 3) mask_lds[buf * kBwdThreads + threadIdx.x] = r.mask;
+        if constexpr (kDrop == 3)
+            mask_lds[buf * kBwdThreads + (threadIdx.x & ~63) + row_slot(threadIdx.x & 63)] = r.mask;
     };
     auto tile_fast = [&](int t) __attribute__((always_inline)) {
         const int i0 = t * kBwdBM;
@@ -259,7 +229,8 @@ __global__ __launch_bounds__(kBwdThreads, (bwd_two_per_cu(DPAD, kDrop, KB) ? 2 :
 #pragma unroll
         for (int t = 0; t < DK; ++t) {
             const bool keep = key[kb] < a.sk && 16 * t + 8 * g < a.d;
-            kf[kb][t] = __builtin_bit_cast(frag_t, keep_or_zero(k_raw[kb][t], keep));
+            // K times scale * log2(e), once: the scores leave the matrix pipe in log2 units
+            kf[kb][t] = scale_frag<T>(keep_or_zero(k_raw[kb][t], keep), a.scale_log2);
             vf[kb][t] = __builtin_bit_cast(frag_t, keep_or_zero(v_raw[kb][t], keep));
         }
     if (t_lo < t_hi) stage_tile(regs, t_lo);
@@ -286,10 +257,15 @@ __global__ __launch_bounds__(kBwdThreads, (bwd_two_per_cu(DPAD, kDrop, KB) ? 2 :
     // S = Q_h K_w^T, dP = dO_h V_w^T: every Q / dO fragment read feeds KB matrix instructions
     auto half_sp = [&](const T* qt, const T* gt, const float* lse_h, const float* delta_h, int hf,
                        f32x16_t (&s)[KB], f32x16_t (&dp)[KB]) __attribute__((always_inline)) {
+        f32x16_t s_init, dp_init;
 #pragma unroll
-        for (int kb = 0; kb < KB; ++kb)
+        for (int r4 = 0; r4 < 4; ++r4) {
+            const f32x4_t l4 = *reinterpret_cast<const f32x4_t*>(lse_h + quad_slot(r4, g));
+            f32x4_t d4 = {0.f, 0.f, 0.f, 0.f};
+            if constexpr (kDrop == 0) d4 = *reinterpret_cast<const f32x4_t*>(delta_h + quad_slot(r4, g));
 #pragma unroll
-            for (int r = 0; r < 16; ++r) s[kb][r] = 0.f, dp[kb][r] = 0.f;
+            for (int e = 0; e < 4; ++e) s_init[4 * r4 + e] = l4[e], dp_init[4 * r4 + e] = d4[e];
+        }
         const T* qrow = qt + 32 * hf * kPitch + a_off;
         const T* grow = gt + 32 * hf * kPitch + a_off;
 #pragma unroll
@@ -298,19 +274,8 @@ __global__ __launch_bounds__(kBwdThreads, (bwd_two_per_cu(DPAD, kDrop, KB) ? 2 :
             const frag_t ga = lds_frag<T>(grow + 16 * x);
 #pragma unroll
             for (int kb = 0; kb < KB; ++kb) {
-                s[kb] = Mma<T>::mma32(qa, kf[kb][x], s[kb]);
-                dp[kb] = Mma<T>::mma32(ga, vf[kb][x], dp[kb]);
-            }
-        }
-        if constexpr (kFold) {
-            // A-operand row of this lane is query pi(c_loc) of the half
-            const frag_t lse_a = row_term(lse_h[pi_row(c_loc)]);
-#pragma unroll
-            for (int kb = 0; kb < KB; ++kb) s[kb] = Mma<T>::mma32(lse_a, ones_f, s[kb]);
-            if constexpr (kDrop == 0) {
-                const frag_t del_a = row_term(delta_h[pi_row(c_loc)]);
-#pragma unroll
-                for (int kb = 0; kb < KB; ++kb) dp[kb] = Mma<T>::mma32(del_a, ones_f, dp[kb]);
+                s[kb] = Mma<T>::mma32(qa, kf[kb][x], x == 0 ? s_init : s[kb]);
+                dp[kb] = Mma<T>::mma32(ga, vf[kb][x], x == 0 ? dp_init : dp[kb]);
             }
         }
     };
@@ -319,49 +284,44 @@ __global__ __launch_bounds__(kBwdThreads, (bwd_two_per_cu(DPAD, kDrop, KB) ? 2 :
     auto half_exp = [&](f32x16_t (&s)[KB], const float* lse_h, int ih0, auto mask_tag)
                         __attribute__((always_inline)) {
         constexpr int kMask = decltype(mask_tag)::value;
-        // register r is query ih0 + 8 g + c with c = acc_row(r, 0); visible iff c_lo <= c <= c_hi
+        // register r is query ih0 + acc_row(r, g) = ih0 + kAccGroupStep g + c with
+        // c = acc_row(r, 0); visible iff c_lo <= c <= c_hi
         int c_lo[KB], c_hi[KB];
 #pragma unroll
         for (int kb = 0; kb < KB; ++kb) {
             c_lo[kb] = 0, c_hi[kb] = 0;
             if constexpr (kMask != 0) {
-                c_lo[kb] = (key[kb] < a.sk) ? (a.causal ? key[kb] - ih0 - 8 * g : -1) : 64;
-                if constexpr (kMask == 2) c_hi[kb] = key[kb] + a.window - 1 - ih0 - 8 * g;
+                c_lo[kb] = (key[kb] < a.sk)
+                               ? (a.causal ? key[kb] - ih0 - kAccGroupStep * g : -1)
+                               : 64;
+                if constexpr (kMask == 2)
+                    c_hi[kb] = key[kb] + a.window - 1 - ih0 - kAccGroupStep * g;
             }
         }
 #pragma unroll
-        for (int r4 = 0; r4 < 4; ++r4) {
-            const int qoff = acc_row(4 * r4, g);
-            f32x4_t lse4 = {0.f, 0.f, 0.f, 0.f};
-            if constexpr (!kFold) lse4 = *reinterpret_cast<const f32x4_t*>(lse_h + qoff);
+        for (int r = 0; r < 16; ++r) {
 #pragma unroll
-            for (int kb = 0; kb < KB; ++kb)
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    float x;
-                    if constexpr (kFold)
-                        x = s[kb][4 * r4 + e] * c_log2;  // lse already subtracted
-                    else
-                        x = __builtin_fmaf(s[kb][4 * r4 + e], c_log2, -lse4[e]);
-                    if constexpr (kBias == 2) {
-                        x += bias_k[kb];
-                    } else if constexpr (kBias == 1) {
-                        const int i = ih0 + qoff + e;
-                        if (i < a.sq && key[kb] < a.sk)
-                            x += a.bias[b * a.bs[0] + h * a.bs[1] + (int64_t)i * a.bs[2] +
-                                        (int64_t)key[kb] * a.bs[3]] * kLog2e;
-                    }
-                    float p = fast_exp2(x);
-                    if constexpr (kMask != 0) {
-                        const int c = acc_row(4 * r4, 0) + e;
-                        if constexpr (kMask == 2) {
-                            if (c < c_lo[kb] || c > c_hi[kb]) p = 0.f;
-                        } else {
-                            if (c < c_lo[kb]) p = 0.f;
-                        }
-                    }
-                    s[kb][4 * r4 + e] = p;
+            for (int kb = 0; kb < KB; ++kb) {
+                float x = s[kb][r];  // scale and lse are in already
+                if constexpr (kBias == 2) {
+                    x += bias_k[kb];
+                } else if constexpr (kBias == 1) {
+                    const int i = ih0 + acc_row(r, g);
+                    if (i < a.sq && key[kb] < a.sk)
+                        x += bias_log2(a.bias[b * a.bs[0] + h * a.bs[1] + (int64_t)i * a.bs[2] +
+                                              (int64_t)key[kb] * a.bs[3]]);
                 }
+                float p = fast_exp2(x);
+                if constexpr (kMask != 0) {
+                    const int c = acc_row(r, 0);
+                    if constexpr (kMask == 2) {
+                        if (c < c_lo[kb] || c > c_hi[kb]) p = 0.f;
+                    } else {
+                        if (c < c_lo[kb]) p = 0.f;
+                    }
+                }
+                s[kb][r] = p;
+            }
         }
     };
     // Keep-bits of one key block of a half tile: wq[e] bit 4 * r4 belongs to register 4 * r4 + e.
@@ -371,7 +331,7 @@ __global__ __launch_bounds__(kBwdThreads, (bwd_two_per_cu(DPAD, kDrop, KB) ? 2 :
         if constexpr (kDrop == 3) {
 #pragma unroll
             for (int r4 = 0; r4 < 4; ++r4) {
-                const u32x4_t w = *reinterpret_cast<const u32x4_t*>(mask_h + acc_row(4 * r4, g));
+                const u32x4_t w = *reinterpret_cast<const u32x4_t*>(mask_h + quad_slot(r4, g));
                 wq[0] |= ((w.x >> c_loc) & 1u) << (4 * r4);
                 wq[1] |= ((w.y >> c_loc) & 1u) << (4 * r4);
                 wq[2] |= ((w.z >> c_loc) & 1u) << (4 * r4);
@@ -385,7 +345,7 @@ __global__ __launch_bounds__(kBwdThreads, (bwd_two_per_cu(DPAD, kDrop, KB) ? 2 :
             uint32_t mine = 0;
 #pragma unroll
             for (int r4 = 0; r4 < 4; ++r4) {
-                const int i = ih0 + acc_row(4 * r4, g) + qpos;
+                const int i = ih0 + acc_row(4 * r4 + qpos, g);
                 if (i < a.sq && kcol < a.sk) {
                     const uint64_t el =
                         ((uint64_t)bh * a.sq + (uint64_t)i) * (uint64_t)a.sk + (uint64_t)(kcol & ~3);
@@ -424,10 +384,9 @@ __global__ __launch_bounds__(kBwdThreads, (bwd_two_per_cu(DPAD, kDrop, KB) ? 2 :
         }
 #pragma unroll
         for (int r4 = 0; r4 < 4; ++r4) {
-            const int qoff = acc_row(4 * r4, g);
-            f32x4_t del4 = {0.f, 0.f, 0.f, 0.f};  // folded and no dropout: already subtracted
-            if constexpr (kDrop != 0 || !kFold)
-                del4 = *reinterpret_cast<const f32x4_t*>(delta_h + qoff);
+            f32x4_t del4 = {0.f, 0.f, 0.f, 0.f};  // no dropout: already subtracted
+            if constexpr (kDrop != 0)
+                del4 = *reinterpret_cast<const f32x4_t*>(delta_h + quad_slot(r4, g));
 #pragma unroll
             for (int kb = 0; kb < KB; ++kb) {
                 float pv[4], dv[4];
@@ -647,16 +606,9 @@ int launch(const AttnArgs& a, hipStream_t st) {
     const int64_t blocks = (int64_t)n_kt * a.batch * a.heads;
     if (blocks <= 0 || blocks > 0x7FFFFFFF) return SLAPO_ERR_SHAPE;
     auto kern = attn_bwd_kernel<T, DPAD, kBias, kDrop, KB>;
-    if (smem > 48 * 1024) {
-        static bool raised = false;  // per instantiation
-        if (!raised) {
-            if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    (int)smem) != hipSuccess)
-                return SLAPO_ERR_LAUNCH;
-            raised = true;
-        }
-    }
+    static std::atomic<uint64_t> lds_ready{0};  // per instantiation, one bit per device
+    if (allow_dynamic_lds(reinterpret_cast<const void*>(kern), smem, lds_ready) != SLAPO_OK)
+        return SLAPO_ERR_LAUNCH;
     hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kBwdThreads), smem, st, a);
     return check_launch();
 }

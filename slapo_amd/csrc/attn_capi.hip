@@ -128,8 +128,8 @@ void set_bias(AttnArgs* a, const float* bias) {
     a->bias = bias;
     a->has_bias = bias ? 1 : 0;
     a->bias_vec4 = 0;
-    if (bias && a->bs[3] == 1 && a->bs[2] == 0 && aligned16(bias) && a->bs[0] % 4 == 0 &&
-        a->bs[1] % 4 == 0)
+    if (bias && a->bs[3] == 1 && aligned16(bias) && a->bs[0] % 4 == 0 && a->bs[1] % 4 == 0 &&
+        a->bs[2] % 4 == 0)
         a->bias_vec4 = 1;
 }
 

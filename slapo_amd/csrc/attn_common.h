@@ -55,14 +55,22 @@ __device__ __forceinline__ u32x2_t lds_read_tr16(const void* lds_ptr) {
     return __builtin_bit_cast(u32x2_t, v);
 }
 
-// Fragment made of two transposing reads: slots 0..3 from rows r0..r0+3, slots 4..7 from
-// r0+4..r0+7 of a row-major LDS tile with `pitch` elements per row.
+// Fragment made of two transposing reads: slots 0..3 from rows r0, r0+4, r0+8, r0+12 and slots 4..7
+// from the rows one below them (the lane offset of tr_lane_off supplies the row stride of 4; see
+// pi_row for why the four rows of one read are four rows apart).
 template <typename T>
 __device__ __forceinline__ typename Mma<T>::frag lds_frag_tr(const T* tile, int pitch) {
     const u32x2_t lo = lds_read_tr16(tile);
-    const u32x2_t hi = lds_read_tr16(tile + 4 * pitch);
+    const u32x2_t hi = lds_read_tr16(tile + pitch);
     u32x4_t v = {lo.x, lo.y, hi.x, hi.y};
     return __builtin_bit_cast(typename Mma<T>::frag, v);
+}
+// Per-lane element offset of such a fragment inside a block of 16 tile rows whose columns
+// 32 x .. 32 x + 31 form the 32 rows of the A operand: lane-group g starts at row 2 g, the four
+// source lanes of a column quad are four rows apart, 16-lane block b takes columns 16 b ..
+__device__ __forceinline__ int tr_lane_off(int lane, int pitch) {
+    return (2 * (lane >> 5) + 4 * ((lane & 15) >> 2)) * pitch + ((lane >> 4) & 1) * 16 +
+           4 * (lane & 3);
 }
 
 template <typename T>
@@ -71,15 +79,31 @@ __device__ __forceinline__ typename Mma<T>::frag lds_frag(const T* p) {
 }
 
 // Row permutation applied when a 32-row A operand is gathered: MFMA row rho takes data row
-// pi(rho), pi = swap of bits 2 and 3.  With it, accumulator registers 8*h .. 8*h+7 of lane-group
-// g hold the eight CONSECUTIVE data rows 16*h + 8*g .. +7, i.e. they form, in order, the k-slots
-// of a B operand for the next MFMA.
+// pi(rho).  Accumulator register r of lane-group g is MFMA row 8 (r / 4) + 4 g + r % 4; with
+// rho = [h][u][g][e1 e0] (bits 4..0) the data row is [h][e1 e0][g][u].  Two properties follow:
+//  * registers 8 h .. 8 h + 7 of lane-group g are, in order, the eight k-slots of a B operand of
+//    the next MFMA whose A operand comes from transposing LDS reads of the same tile;
+//  * the four k-slots of one transposing read (e = 0..3) are data rows FOUR apart.  With a row
+//    pitch of DPAD + 8 elements four rows are 64 bytes (mod 256) apart, so the 4 rows x 64 bytes
+//    that 32 lanes read in one LDS cycle fall into 64 different banks.  With consecutive rows
+//    the same reads collide two-fold at head_dim 64 / 96 and four-fold at 128 (measured: 437 and
+//    851 ns against 247 ns per 128 KB and CU).
 __device__ __forceinline__ int pi_row(int rho) {
-    return (rho & ~0xC) | ((rho & 4) << 1) | ((rho & 8) >> 1);
+    return (rho & 16) | ((rho & 3) << 2) | (((rho >> 2) & 1) << 1) | ((rho >> 3) & 1);
 }
 // Data row (0..31) held by accumulator register r of lane-group g under that permutation.
 __device__ __forceinline__ constexpr int acc_row(int r, int g) {
-    return ((r >> 3) << 4) + (g << 3) + (((r >> 2) & 1) << 2) + (r & 3);
+    return ((r >> 3) << 4) + ((r & 3) << 2) + (g << 1) + ((r >> 2) & 1);
+}
+constexpr int kAccGroupStep = 2;  // acc_row(r, g) = acc_row(r, 0) + kAccGroupStep * g
+// Per-row values (bias, lse, delta, keep words) of a 32-row block are kept in LDS at position
+// row_slot(row), so that ONE 128-bit read at quad_slot(r4, g) returns the values of registers
+// 4 r4 .. 4 r4 + 3 of lane-group g in order.
+__device__ __forceinline__ constexpr int row_slot(int row) {
+    return (row & ~15) | ((row & 3) << 2) | ((row >> 2) & 3);
+}
+__device__ __forceinline__ constexpr int quad_slot(int r4, int g) {
+    return ((r4 >> 1) << 4) + (g << 3) + ((r4 & 1) << 2);
 }
 
 // Two floats -> one packed register of T, round to nearest even (v_cvt_pk_{f16,bf16}_f32).
@@ -93,6 +117,38 @@ __device__ __forceinline__ uint32_t pack2(float a, float b) {
 }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// acc + lo + hi of a packed pair of T, in fp32 (v_dot2c_f32_{f16,bf16} against a pair of ones).
+template <typename T>
+__device__ __forceinline__ float sum2(uint32_t pair, float acc);
+template <>
+__device__ __forceinline__ float sum2<f16_t>(uint32_t pair, float acc) {
+    const f16x2_t ones = {(f16_t)1.f, (f16_t)1.f};
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, pair), ones, acc, false);
+}
+template <>
+__device__ __forceinline__ float sum2<bf16_t>(uint32_t pair, float acc) {
+    const bf16x2_t ones = {(bf16_t)1.f, (bf16_t)1.f};
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pair), ones, acc, false);
+}
+
+// An additive bias in log2 units.  Mask values near the most negative finite number (HF-style
+// padding masks use finfo.min) would overflow to -inf under the multiplication; they stay
+// finite, so that a row that sees only such keys keeps a finite, uniform softmax as in the
+// reference.  A true -inf is left alone.
+__device__ __forceinline__ float bias_log2(float b) {
+    const float v = b * kLog2e;
+    return (v == -INFINITY && b != -INFINITY) ? -3.4028234663852886e38f : v;
+}
+
+// Fragment of 8 elements times a scalar, rounded back to T.
+template <typename T>
+__device__ __forceinline__ typename Mma<T>::frag scale_frag(u32x4_t raw, float c) {
+    typename Mma<T>::frag f = __builtin_bit_cast(typename Mma<T>::frag, raw);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) f[j] = (T)((float)f[j] * c);
+    return f;
+}
 
 // Exchange with lane l ^ 32 through v_permlane32_swap (upper half of the first register <-> lower
 // half of the second).  Starting from two copies of v, the first register ends up holding the lower

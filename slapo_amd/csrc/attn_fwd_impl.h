@@ -101,10 +101,12 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
                                                          min(16 * t + 8 * g, a.d - 8));
         ks.load_indexed(k_base, a.ks[1], t_lo * kBN, a.sk, a.d);
         vs.load_indexed(v_base, a.vs[1], t_lo * kBN, a.sk, a.d);
+        // Q is multiplied by scale * log2(e) once, here: the scores leave the matrix pipe in log2
+        // units and no per-score multiplication is left in the tile body.
 #pragma unroll
         for (int t = 0; t < DK; ++t)
-            qf[t] = __builtin_bit_cast(
-                frag_t, keep_or_zero(q_raw[t], q_row < a.sq && 16 * t + 8 * g < a.d));
+            qf[t] = scale_frag<T>(keep_or_zero(q_raw[t], q_row < a.sq && 16 * t + 8 * g < a.d),
+                                  a.scale_log2);
     }
 
     f32x16_t o_acc[DV];
@@ -112,16 +114,23 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
     for (int x = 0; x < DV; ++x)
 #pragma unroll
         for (int r = 0; r < 16; ++r) o_acc[x][r] = 0.f;
-    // Without a bias the scores stay in units of the raw dot product and the scale is folded
-    // into the exponential's FMA; with a bias they are converted to log2 units when the bias is
-    // added.  m_run is the reference in score units, m_ref = m_run in log2 units (0 if -inf).
+    // Softmax state of this lane's query, in log2 units (Q carries scale * log2(e)):
+    //   m_run  reference point of l_run / o_acc (-inf: nothing accumulated yet);
+    //   m_ref  the part of it that the matrix pipe subtracts: the score accumulators start from
+    //          neg_m = -m_ref in all sixteen registers, so a tile's scores arrive as s - m_ref and
+    //          go straight into exp2.  m_ref == m_run while m_run is an ordinary number.  A row
+    //          that has met nothing but keys masked with a huge negative bias has m_run below
+    //          kHugeNeg; subtracting that inside the accumulator would swallow the scores of the
+    //          first real key, so m_ref stays 0 there and such rows take the slow path.
+    constexpr float kHugeNeg = -1e30f;
     float m_run = -INFINITY;
     float m_ref = 0.f;
     float l_run = 0.f;  // this lane's share of the running sum
+    f32x16_t neg_m;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) neg_m[r] = 0.f;
 
     const int wq_last = min(wq0 + 31, a.sq - 1);
-    const float c_log2 = a.scale_log2;
-    const float slack = kBias ? kMaxSlack : kMaxSlack / c_log2;
     uint64_t drop_row_base = 0;
     if constexpr (kDrop != 0)
         drop_row_base = ((uint64_t)bh * a.sq + (uint64_t)q_row) * (uint64_t)a.sk;
@@ -138,14 +147,14 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
             bias_stage = bias_keys[(int64_t)min(j0 + lane, a.sk - 1) * a.bs[3]];
     };
     auto store_bias = [&](int slot) __attribute__((always_inline)) {
-        if constexpr (kBias == 2) bias_lds[slot * kBN + lane] = bias_stage * kLog2e;
+        if constexpr (kBias == 2) bias_lds[slot * kBN + row_slot(lane)] = bias_log2(bias_stage);
     };
     const float* bias_tile = bias_lds;  // the slot of the tile in process
     request_bias(t_lo * kBN);
 
     // per-lane LDS offsets (elements) that do not change from tile to tile
     const int k_off = pi_row(i_loc) * kPitch + 8 * g;
-    const int v_off = (8 * g + ((lane & 15) >> 2)) * kPitch + ((lane >> 4) & 1) * 16 + 4 * (lane & 3);
+    const int v_off = tr_lane_off(lane, kPitch);
 
     // Wavefront-uniform: does tile t hold any visible key for this wavefront's queries?
     auto tile_active = [&](int t) __attribute__((always_inline)) {
@@ -161,12 +170,11 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
                (a.window > 0 && wq_last - j0 >= a.window);
     };
 
-    // S^T half = K_half Q^T
+    // S^T half = K_half Q^T - m_ref (the accumulator starts from neg_m)
     auto half_scores = [&](const T* kt, int kb, f32x16_t& s) __attribute__((always_inline)) {
+        s = Mma<T>::mma32(lds_frag<T>(kt + kb * 32 * kPitch + k_off), qf[0], neg_m);
 #pragma unroll
-        for (int r = 0; r < 16; ++r) s[r] = 0.f;
-#pragma unroll
-        for (int x = 0; x < DK; ++x)
+        for (int x = 1; x < DK; ++x)
             s = Mma<T>::mma32(lds_frag<T>(kt + kb * 32 * kPitch + k_off + 16 * x), qf[x], s);
     };
     // bias, masks and maximum of one half; mask_tag: 0 = every key visible, 1 = upper bound only
@@ -175,42 +183,49 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
                            __attribute__((always_inline)) -> float {
         constexpr int kMask = decltype(mask_tag)::value;
         const int j0 = t * kBN + 32 * kb;
-        // register r is key j0 + 8 g + c with c = acc_row(r, 0); visible iff c_lo <= c <= c_hi
+        // register r is key j0 + acc_row(r, g) = j0 + kAccGroupStep g + c with c = acc_row(r, 0);
+        // visible iff c_lo <= c <= c_hi
         int c_lo = 0, c_hi = 0;
         if constexpr (kMask != 0) {
             const int k_max = a.causal ? min(a.sk - 1, q_row) : a.sk - 1;
-            c_hi = k_max - j0 - 8 * g;
-            if constexpr (kMask == 2) c_lo = q_row - a.window + 1 - j0 - 8 * g;
+            c_hi = k_max - j0 - kAccGroupStep * g;
+            if constexpr (kMask == 2) c_lo = q_row - a.window + 1 - j0 - kAccGroupStep * g;
+        }
+        if constexpr (kBias == 1) {
+            // Registers 8 h + e and 8 h + 4 + e are keys 2 g and 2 g + 1 of the aligned group of
+            // four keys at j0 + 16 h + 4 e: one 16-byte read per group where the layout allows.
+#pragma unroll
+            for (int he = 0; he < 8; ++he) {
+                const int kg = j0 + 16 * (he >> 2) + 4 * (he & 3);
+                float b_lo = 0.f, b_hi = 0.f;
+                if (a.bias_vec4 && kg + 3 < a.sk) {
+                    const f32x4_t t4 = *reinterpret_cast<const f32x4_t*>(bias_row + kg);
+                    b_lo = g ? t4.z : t4.x;
+                    b_hi = g ? t4.w : t4.y;
+                } else {
+                    const int k_lo = kg + 2 * g;
+                    if (k_lo < a.sk) b_lo = bias_row[(int64_t)k_lo * a.bs[3]];
+                    if (k_lo + 1 < a.sk) b_hi = bias_row[(int64_t)(k_lo + 1) * a.bs[3]];
+                }
+                s[8 * (he >> 2) + (he & 3)] += bias_log2(b_lo);
+                s[8 * (he >> 2) + 4 + (he & 3)] += bias_log2(b_hi);
+            }
         }
         float mx = -INFINITY;
 #pragma unroll
         for (int r4 = 0; r4 < 4; ++r4) {
             if constexpr (kBias == 2) {
                 const f32x4_t t4 = *reinterpret_cast<const f32x4_t*>(bias_tile + 32 * kb +
-                                                                     acc_row(4 * r4, g));
-                s[4 * r4 + 0] = __builtin_fmaf(s[4 * r4 + 0], c_log2, t4.x);
-                s[4 * r4 + 1] = __builtin_fmaf(s[4 * r4 + 1], c_log2, t4.y);
-                s[4 * r4 + 2] = __builtin_fmaf(s[4 * r4 + 2], c_log2, t4.z);
-                s[4 * r4 + 3] = __builtin_fmaf(s[4 * r4 + 3], c_log2, t4.w);
-            } else if constexpr (kBias == 1) {
-                const int key0 = j0 + acc_row(4 * r4, g);
-                float bv[4] = {0.f, 0.f, 0.f, 0.f};
-                if (a.bias_vec4 && key0 + 3 < a.sk) {
-                    const f32x4_t t4 = *reinterpret_cast<const f32x4_t*>(bias_row + key0);
-                    bv[0] = t4.x, bv[1] = t4.y, bv[2] = t4.z, bv[3] = t4.w;
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 4; ++e)
-                        if (key0 + e < a.sk) bv[e] = bias_row[(int64_t)(key0 + e) * a.bs[3]];
-                }
-#pragma unroll
-                for (int e = 0; e < 4; ++e)
-                    s[4 * r4 + e] = __builtin_fmaf(s[4 * r4 + e], c_log2, bv[e] * kLog2e);
+                                                                     quad_slot(r4, g));
+                s[4 * r4 + 0] += t4.x;
+                s[4 * r4 + 1] += t4.y;
+                s[4 * r4 + 2] += t4.z;
+                s[4 * r4 + 3] += t4.w;
             }
             if constexpr (kMask != 0) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    const int c = acc_row(4 * r4, 0) + e;
+                    const int c = acc_row(4 * r4 + e, 0);
                     if constexpr (kMask == 2) {
                         if (c > c_hi || c < c_lo) s[4 * r4 + e] = -INFINITY;
                     } else {
@@ -223,47 +238,55 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
         }
         return mx;
     };
-    // move the reference point if this tile's maximum calls for it (rare after the first tile)
-    auto update_reference = [&](float mx) __attribute__((always_inline)) {
-        const bool move = (mx > m_run + slack || m_run == -INFINITY) && mx != -INFINITY;
+    // Moves the reference point if this tile's maximum (mx, relative to m_ref) calls for it and
+    // re-bases the tile's scores.  Rare after a row's first tile.
+    auto update_reference = [&](float mx, f32x16_t& s0, f32x16_t& s1)
+                                __attribute__((always_inline)) {
+        const bool ordinary = m_run > kHugeNeg;
+        const bool move = (mx > kMaxSlack || !ordinary) && mx != -INFINITY;
         if (__builtin_expect(__builtin_amdgcn_ballot_w64(move) != 0, 0)) {
-            const float m_new = move ? mx : m_run;
-            const float m_new_ref = kBias ? m_new : m_new * c_log2;
+            const float mx_abs = mx + m_ref;
+            const float new_run = ordinary ? mx_abs : fmaxf(m_run, mx_abs);
             // exp2(old reference - new reference); an unset reference (-inf) scales by 0
-            const float alpha = (m_run == -INFINITY) ? 0.f : fast_exp2(m_ref - m_new_ref);
+            const float alpha = (m_run == -INFINITY) ? 0.f : fast_exp2(m_run - new_run);
             if (move) {
-                m_run = m_new;
-                m_ref = m_new_ref;
+                const float sub = ordinary ? mx : new_run - m_ref;
+                m_run = new_run;
+                m_ref = new_run > kHugeNeg ? new_run : 0.f;
                 l_run *= alpha;
 #pragma unroll
                 for (int x = 0; x < DV; ++x)
 #pragma unroll
                     for (int r = 0; r < 16; ++r) o_acc[x][r] *= alpha;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    s0[r] -= sub;
+                    s1[r] -= sub;
+                    neg_m[r] = -m_ref;
+                }
             }
         }
     };
-    // probabilities of one half: exp2, row sum, dropout, pack to T
+    // probabilities of one half: exp2, dropout, pack to T, row sum
     // (drop_bits: the keep bits of this lane's 16 keys at their position in the half)
     auto half_prob = [&](f32x16_t& s, int t, int kb, uint32_t (&pw)[8], uint32_t& drop_bits)
                          __attribute__((always_inline)) {
-        float psum = 0.f;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            float p;
-            if constexpr (kBias)
-                p = fast_exp2(s[r] - m_ref);
-            else
-                p = fast_exp2(__builtin_fmaf(s[r], c_log2, -m_ref));
-            s[r] = p;
-            psum += p;
-        }
-        l_run += psum;
+        for (int r = 0; r < 16; ++r) s[r] = fast_exp2(s[r]);
         if constexpr (kDrop != 0) {
-            const int j0 = t * kBN + 32 * kb;
-            uint32_t mine = 0;  // keep bits of this lane's 16 keys, at their position in the half
+            float psum = 0.f;
 #pragma unroll
-            for (int r4 = 0; r4 < 4; ++r4) {
-                const int key0 = j0 + acc_row(4 * r4, g);
+            for (int r = 0; r < 16; ++r) psum += s[r];
+            l_run += psum;
+            // Philox blocks cover four consecutive keys; the two lanes of a query (l, l ^ 32)
+            // draw the blocks of keys 8 g .. 8 g + 7 of each 16-key group and exchange them.  The
+            // combined word (bit j = key j of the half) is also what the backward reads.
+            const int j0 = t * kBN + 32 * kb;
+            uint32_t mine = 0;
+#pragma unroll
+            for (int blk = 0; blk < 4; ++blk) {
+                const int pos = 16 * (blk >> 1) + 8 * g + 4 * (blk & 1);
+                const int key0 = j0 + pos;
                 uint32_t bits = 0;
                 if (q_row < a.sq && key0 < a.sk) {
                     const uint64_t e0 = drop_row_base + (uint64_t)key0;
@@ -272,17 +295,26 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
                     else
                         bits = dropout_keep_any(a.rng, e0, min(4, a.sk - key0));
                 }
-                mine |= bits << acc_row(4 * r4, g);
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const float p = s[4 * r4 + e];
-                    s[4 * r4 + e] = ((bits >> e) & 1u) ? p * a.rng.inv_keep : 0.f;
-                }
+                mine |= bits << pos;
             }
-            drop_bits = mine;
-        }
+            mine = or_xor32(mine);
+            const uint32_t mine_g = mine >> (kAccGroupStep * g);
 #pragma unroll
-        for (int r2 = 0; r2 < 8; ++r2) pw[r2] = pack2<T>(s[2 * r2], s[2 * r2 + 1]);
+            for (int r = 0; r < 16; ++r)
+                s[r] = ((mine_g >> acc_row(r, 0)) & 1u) ? s[r] * a.rng.inv_keep : 0.f;
+            drop_bits = mine;
+#pragma unroll
+            for (int r2 = 0; r2 < 8; ++r2) pw[r2] = pack2<T>(s[2 * r2], s[2 * r2 + 1]);
+        } else {
+            // Without dropout the row sum is taken over the rounded probabilities, two per
+            // instruction (v_dot2c_f32_{f16,bf16} against a pair of ones): the normaliser then
+            // belongs to exactly the numbers that multiply V.
+#pragma unroll
+            for (int r2 = 0; r2 < 8; ++r2) {
+                pw[r2] = pack2<T>(s[2 * r2], s[2 * r2 + 1]);
+                l_run = sum2<T>(pw[r2], l_run);
+            }
+        }
     };
     // O^T += V_half^T P_half^T
     auto half_accumulate = [&](const T* vt, int kb, const uint32_t (&pw)[8])
@@ -306,7 +338,7 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
         half_scores(kt, 1, s1);
         const float mx =
             max_xor32(fmaxf(finish_half(s0, t, 0, mask_tag), finish_half(s1, t, 1, mask_tag)));
-        update_reference(mx);
+        update_reference(mx, s0, s1);
         uint32_t bits0 = 0, bits1 = 0;
         half_prob(s0, t, 0, pw0, bits0);
         half_accumulate(vt, 0, pw0);
@@ -318,7 +350,7 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
         // with the matrix instructions (10 % of the forward).
         if constexpr (kDrop != 0) {
             if (a.keep_mask != nullptr) {
-                const uint32_t w0 = or_xor32(bits0), w1 = or_xor32(bits1);
+                const uint32_t w0 = bits0, w1 = bits1;  // already combined over the lane pair
                 uint32_t* row = a.keep_mask +
                                 ((int64_t)bh * a.mask_words + 2 * t) * a.mask_pitch + q_row;
                 if (g == 0 && q_row < a.sq) {
@@ -422,10 +454,13 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
                     *reinterpret_cast<u32x2_t*>(o_row + d0) = w;
                 }
             }
-        if (g == 0) {
-            const float m_log2 = (m_run == -INFINITY) ? -INFINITY : m_ref;
-            a.lse[(int64_t)bh * a.sq + q_row] = (m_log2 + __builtin_log2f(l_tot)) * kLn2;
-        }
+        // A row that met nothing but keys masked with a huge negative bias has a uniform softmax
+        // here (as in the reference) but no log-sum-exp that fp32 can hold next to its scores:
+        // +inf is stored, which makes the backward treat the row as contributing no gradient.
+        if (g == 0)
+            a.lse[(int64_t)bh * a.sq + q_row] = (m_run > kHugeNeg || m_run == -INFINITY)
+                                                    ? (m_run + __builtin_log2f(l_tot)) * kLn2
+                                                    : INFINITY;
     }
 }
 
@@ -438,16 +473,9 @@ int launch(const AttnArgs& a, hipStream_t st) {
     const int64_t blocks = (int64_t)n_qt * a.batch * a.heads;
     if (blocks <= 0 || blocks > 0x7FFFFFFF) return SLAPO_ERR_SHAPE;
     auto kern = attn_fwd_kernel<T, DPAD, kBias, kDrop, kWin>;
-    if (smem > 48 * 1024) {
-        static bool raised = false;  // per instantiation
-        if (!raised) {
-            if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize,
-                                    (int)smem) != hipSuccess)
-                return SLAPO_ERR_LAUNCH;
-            raised = true;
-        }
-    }
+    static std::atomic<uint64_t> lds_ready{0};  // per instantiation, one bit per device
+    if (allow_dynamic_lds(reinterpret_cast<const void*>(kern), smem, lds_ready) != SLAPO_OK)
+        return SLAPO_ERR_LAUNCH;
     hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kThreads), smem, st, a);
     return check_launch();
 }

@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/slapo_amd.h"
 #include "philox.h"
 
@@ -78,6 +80,21 @@ __device__ __forceinline__ void store_packet_nt(T* p, const Packet<T>& r) {
 inline int check_launch() {
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? SLAPO_OK : SLAPO_ERR_LAUNCH;
+}
+
+// Kernels that need more than 48 KB of dynamic LDS must be told so once per device.  `done` is
+// the caller's flag word (one per kernel instantiation), bit i = device i has been set up.
+inline int allow_dynamic_lds(const void* kern, size_t bytes, std::atomic<uint64_t>& done) {
+    if (bytes <= 48 * 1024) return SLAPO_OK;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return SLAPO_ERR_LAUNCH;
+    const uint64_t bit = 1ull << (dev & 63);
+    if (dev < 64 && (done.load(std::memory_order_acquire) & bit)) return SLAPO_OK;
+    if (hipFuncSetAttribute(kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes) !=
+        hipSuccess)
+        return SLAPO_ERR_LAUNCH;
+    if (dev < 64) done.fetch_or(bit, std::memory_order_release);
+    return SLAPO_OK;
 }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
