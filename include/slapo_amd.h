@@ -6,7 +6,8 @@
  * leaves Python for a fused kernel are third-party calls.  Every entry point below names the
  * reference call site whose callee it replaces.  All entry points
  *   - take plain device pointers, sizes, strides and a hipStream_t passed as void*;
- *   - never allocate or free memory (workspaces are caller-provided);
+ *   - never allocate or free memory (workspaces are caller-provided, except for
+ *     slapo_amd_attn_bwd_static_scratch, whose workspace is an array inside the library);
  *   - are stateless and re-entrant; they enqueue work on `stream` and return without
  *     synchronising;
  *   - return 0 on success or a negative SLAPO_ERR_* code (see slapo_amd_status_string).
@@ -265,6 +266,21 @@ int slapo_amd_attn_bwd_stages(const slapo_attn_params* prm, const void* q, const
                               const int64_t dq_strides[3], const int64_t dk_strides[3],
                               const int64_t dv_strides[3], void* workspace,
                               size_t workspace_bytes, int stages, void* stream);
+
+/* slapo_amd_attn_bwd without the workspace arguments.  No counterpart in the reference: it is
+ * for callers that cannot allocate (code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc).  delta is kept in a 4 MiB array inside the library, one copy per device,
+ * held until the process ends; the call itself allocates and frees nothing.  Limit:
+ * batch * heads * seqlen_q <= 1 048 576, else SLAPO_ERR_WORKSPACE.  All calls on one device share
+ * the array (every call overwrites the part it reads, so nothing has to be cleared): calls that
+ * overlap in time on one device, on any streams, race.  Results are bitwise those of
+ * slapo_amd_attn_bwd. */
+int slapo_amd_attn_bwd_static_scratch(const slapo_attn_params* prm, const void* q, const void* k,
+                                      const void* v, const float* bias, const void* o,
+                                      const void* dout, const float* lse, void* dq, void* dk,
+                                      void* dv, const int64_t dq_strides[3],
+                                      const int64_t dk_strides[3], const int64_t dv_strides[3],
+                                      void* stream);
 
 #ifdef __cplusplus
 }

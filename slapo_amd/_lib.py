@@ -132,6 +132,11 @@ PROTOTYPES = {
          ctypes.POINTER(c_i64), ctypes.POINTER(c_i64), ctypes.POINTER(c_i64), c_vp,
          ctypes.c_size_t, c_vp],
     ),
+    "slapo_amd_attn_bwd_static_scratch": (
+        ctypes.c_int,
+        [ctypes.POINTER(AttnParams), c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp,
+         ctypes.POINTER(c_i64), ctypes.POINTER(c_i64), ctypes.POINTER(c_i64), c_vp],
+    ),
     "slapo_amd_attn_bwd_stages": (
         ctypes.c_int,
         [ctypes.POINTER(AttnParams), c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp, c_vp,

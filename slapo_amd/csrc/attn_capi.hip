@@ -1,6 +1,8 @@
 // C-ABI entry points of the attention path: argument validation, kernel selection (MFMA kernels
 // for fp16 / bf16, FMA kernels for fp32) and the small helper kernels around the backward
 // (delta = rowsum(dO * O)).
+#include <mutex>
+
 #include "attn_common.h"
 
 namespace slapo {
@@ -246,5 +248,51 @@ extern "C" int slapo_amd_attn_bwd(const slapo_attn_params* prm, const void* q, c
                                   void* workspace, size_t workspace_bytes, void* stream) {
     return slapo_amd_attn_bwd_stages(prm, q, k, v, bias, o, dout, lse, dq, dk, dv, dq_strides,
                                      dk_strides, dv_strides, workspace, workspace_bytes,
+                                     SLAPO_BWD_ALL, stream);
+}
+
+// ---- backward without a caller workspace -------------------------------------------------------
+// delta = rowsum(dO * O) lives in an array of the library's own, so that callers that must not
+// allocate (HIP graph capture, serving loops) need no workspace: every device that runs the
+// library holds one copy of the array until the process ends.
+namespace {
+
+constexpr size_t kScratchFloats = size_t(1) << 20;  // 4 MiB: batch * heads * seqlen_q <= 1 048 576
+__device__ __align__(256) float scratch[kScratchFloats];
+
+std::mutex scratch_lock;
+float* scratch_of_device[64] = {};  // device address of `scratch`, per device, once resolved
+
+// The array's name is only a handle on the host; its address on the current device comes from
+// the runtime, once per device.
+int scratch_on_current_device(float** out) {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return SLAPO_ERR_DEVICE;
+    std::lock_guard<std::mutex> guard(scratch_lock);
+    if (!scratch_of_device[dev]) {
+        void* p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p)
+            return SLAPO_ERR_DEVICE;
+        scratch_of_device[dev] = static_cast<float*>(p);
+    }
+    *out = scratch_of_device[dev];
+    return SLAPO_OK;
+}
+
+}  // namespace
+
+extern "C" int slapo_amd_attn_bwd_static_scratch(
+    const slapo_attn_params* prm, const void* q, const void* k, const void* v, const float* bias,
+    const void* o, const void* dout, const float* lse, void* dq, void* dk, void* dv,
+    const int64_t dq_strides[3], const int64_t dk_strides[3], const int64_t dv_strides[3],
+    void* stream) {
+    const size_t need = slapo_amd_attn_bwd_workspace_bytes(prm);
+    if (need == 0) return SLAPO_ERR_SHAPE;
+    if (need > kScratchFloats * sizeof(float)) return SLAPO_ERR_WORKSPACE;
+    float* ws = nullptr;
+    const int rc = scratch_on_current_device(&ws);
+    if (rc != SLAPO_OK) return rc;
+    return slapo_amd_attn_bwd_stages(prm, q, k, v, bias, o, dout, lse, dq, dk, dv, dq_strides,
+                                     dk_strides, dv_strides, ws, kScratchFloats * sizeof(float),
                                      SLAPO_BWD_ALL, stream);
 }
