@@ -570,30 +570,19 @@ __global__ __launch_bounds__(kBwdThreads, (bwd_two_per_cu(DPAD, kDrop, KB) ? 2 :
         while (t < t_hi) t += generic_step(t);
     }
     // ---- write dK, dV ----
-#pragma unroll
-    for (int kb = 0; kb < KB; ++kb) {
-        if (key[kb] >= a.sk) continue;
-        T* dk_row =
-            reinterpret_cast<T*>(a.dk) + b * a.dks[0] + (int64_t)key[kb] * a.dks[1] + h * a.dks[2];
-        T* dv_row =
-            reinterpret_cast<T*>(a.dv) + b * a.dvs[0] + (int64_t)key[kb] * a.dvs[1] + h * a.dvs[2];
-#pragma unroll
-        for (int x = 0; x < DV; ++x)
-#pragma unroll
-            for (int r4 = 0; r4 < 4; ++r4) {
-                const int d0 = x * 32 + 8 * r4 + 4 * g;
-                if (d0 < a.d) {
-                    const f32x16_t& ka = dk_acc[kb][x];
-                    const f32x16_t& va = dv_acc[kb][x];
-                    u32x2_t wk, wv;
-                    wk.x = pack2<T>(ka[4 * r4] * a.scale, ka[4 * r4 + 1] * a.scale);
-                    wk.y = pack2<T>(ka[4 * r4 + 2] * a.scale, ka[4 * r4 + 3] * a.scale);
-                    wv.x = pack2<T>(va[4 * r4], va[4 * r4 + 1]);
-                    wv.y = pack2<T>(va[4 * r4 + 2], va[4 * r4 + 3]);
-                    *reinterpret_cast<u32x2_t*>(dk_row + d0) = wk;
-                    *reinterpret_cast<u32x2_t*>(dv_row + d0) = wv;
-                }
-            }
+    // every wavefront is past the last barrier of the loop: the tile buffers are free, and each
+    // wavefront routes its rows through its own part of them (dK through the Q buffers, dV
+    // through the dO buffers)
+    static_assert(KB == 1, "the output staging assumes 32 keys per wavefront");
+    if (kw0 < a.sk) {
+        T* dk_row0 =
+            reinterpret_cast<T*>(a.dk) + b * a.dks[0] + (int64_t)kw0 * a.dks[1] + h * a.dks[2];
+        T* dv_row0 =
+            reinterpret_cast<T*>(a.dv) + b * a.dvs[0] + (int64_t)kw0 * a.dvs[1] + h * a.dvs[2];
+        store_block_via_lds<T, DPAD, kPitch>(dk_acc[0], a.scale, q_lds + wave * 32 * kPitch,
+                                             dk_row0, a.dks[1], a.sk - kw0, a.d);
+        store_block_via_lds<T, DPAD, kPitch>(dv_acc[0], 1.0f, g_lds + wave * 32 * kPitch, dv_row0,
+                                             a.dvs[1], a.sk - kw0, a.d);
     }
 }
 

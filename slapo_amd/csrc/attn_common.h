@@ -260,6 +260,41 @@ __device__ __forceinline__ int padded_key_limit(const AttnArgs& a, int b, int h,
     return limit + 1;
 }
 
+// Writes a wavefront's 32 x d block of results to global memory with full-line stores.  The
+// block arrives transposed in accumulator registers (acc[x][4 r4 + e] of lane (i, g) is element
+// (row i, column 32 x + 8 r4 + 4 g + e)), goes through `wave_lds` (32 rows of PITCH elements that
+// only this wavefront touches) and leaves as 16 bytes per lane, eight or more lanes per row.
+// Storing straight from the registers would write 8 bytes per lane to 32 different rows per
+// instruction: sixteen-byte pieces of 128-byte lines.
+template <typename T, int DPAD, int PITCH>
+__device__ __forceinline__ void store_block_via_lds(const f32x16_t (&acc)[DPAD / 32], float mul,
+                                                    T* wave_lds, T* out_row0, int64_t row_stride,
+                                                    int n_rows, int d) {
+    const int lane = threadIdx.x & 63;
+    const int i = lane & 31, g = lane >> 5;
+#pragma unroll
+    for (int x = 0; x < DPAD / 32; ++x)
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) {
+            u32x2_t w;
+            w.x = pack2<T>(acc[x][4 * r4 + 0] * mul, acc[x][4 * r4 + 1] * mul);
+            w.y = pack2<T>(acc[x][4 * r4 + 2] * mul, acc[x][4 * r4 + 3] * mul);
+            *reinterpret_cast<u32x2_t*>(wave_lds + i * PITCH + 32 * x + 8 * r4 + 4 * g) = w;
+        }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    constexpr int kChunksPerRow = DPAD / 8;
+#pragma unroll
+    for (int pass = 0; pass < 32 * kChunksPerRow / 64; ++pass) {
+        const int idx = pass * 64 + lane;
+        const int row = idx / kChunksPerRow, c = idx % kChunksPerRow;
+        const u32x4_t v = *reinterpret_cast<const u32x4_t*>(wave_lds + row * PITCH + 8 * c);
+        if (row < n_rows && 8 * c < d)
+            *reinterpret_cast<u32x4_t*>(out_row0 + (int64_t)row * row_stride + 8 * c) = v;
+    }
+}
+
 // Stage a [ROWS x DPAD] tile of T (rows row0.., zero beyond n_rows / beyond d) through registers.
 // The global loads are unconditional (out-of-range rows are clamped to the last valid row and
 // zeroed when the tile is written to LDS), so they stay in the caller's basic block and the

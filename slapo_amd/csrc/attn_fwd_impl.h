@@ -114,21 +114,12 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
     for (int x = 0; x < DV; ++x)
 #pragma unroll
         for (int r = 0; r < 16; ++r) o_acc[x][r] = 0.f;
-    // Softmax state of this lane's query, in log2 units (Q carries scale * log2(e)):
-    //   m_run  reference point of l_run / o_acc (-inf: nothing accumulated yet);
-    //   m_ref  the part of it that the matrix pipe subtracts: the score accumulators start from
-    //          neg_m = -m_ref in all sixteen registers, so a tile's scores arrive as s - m_ref and
-    //          go straight into exp2.  m_ref == m_run while m_run is an ordinary number.  A row
-    //          that has met nothing but keys masked with a huge negative bias has m_run below
-    //          kHugeNeg; subtracting that inside the accumulator would swallow the scores of the
-    //          first real key, so m_ref stays 0 there and such rows take the slow path.
+    // Softmax state of this lane's query, in log2 units (Q carries scale * log2(e)): m_run is the
+    // reference point of l_run / o_acc (-inf: nothing accumulated yet), moved lazily.
     constexpr float kHugeNeg = -1e30f;
     float m_run = -INFINITY;
-    float m_ref = 0.f;
+    float m_ref = 0.f;  // what the exponentials subtract: m_run, or 0 while m_run is -inf
     float l_run = 0.f;  // this lane's share of the running sum
-    f32x16_t neg_m;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) neg_m[r] = 0.f;
 
     const int wq_last = min(wq0 + 31, a.sq - 1);
     uint64_t drop_row_base = 0;
@@ -170,11 +161,12 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
                (a.window > 0 && wq_last - j0 >= a.window);
     };
 
-    // S^T half = K_half Q^T - m_ref (the accumulator starts from neg_m)
+    // S^T half = K_half Q^T, in log2 units
     auto half_scores = [&](const T* kt, int kb, f32x16_t& s) __attribute__((always_inline)) {
-        s = Mma<T>::mma32(lds_frag<T>(kt + kb * 32 * kPitch + k_off), qf[0], neg_m);
 #pragma unroll
-        for (int x = 1; x < DK; ++x)
+        for (int r = 0; r < 16; ++r) s[r] = 0.f;
+#pragma unroll
+        for (int x = 0; x < DK; ++x)
             s = Mma<T>::mma32(lds_frag<T>(kt + kb * 32 * kPitch + k_off + 16 * x), qf[x], s);
     };
     // bias, masks and maximum of one half; mask_tag: 0 = every key visible, 1 = upper bound only
@@ -238,32 +230,23 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
         }
         return mx;
     };
-    // Moves the reference point if this tile's maximum (mx, relative to m_ref) calls for it and
-    // re-bases the tile's scores.  Rare after a row's first tile.
-    auto update_reference = [&](float mx, f32x16_t& s0, f32x16_t& s1)
-                                __attribute__((always_inline)) {
-        const bool ordinary = m_run > kHugeNeg;
-        const bool move = (mx > kMaxSlack || !ordinary) && mx != -INFINITY;
+    // Moves the reference point if this tile's maximum calls for it (rare after a row's first
+    // tile): only when the maximum exceeds it by more than kMaxSlack, so that the rescale of the
+    // accumulators stays off the common path.  A row that has met nothing but keys masked with a
+    // huge negative bias sits at that value and moves up to the first real key like any other.
+    auto update_reference = [&](float mx) __attribute__((always_inline)) {
+        const bool move = mx > m_run + kMaxSlack && mx != -INFINITY;
         if (__builtin_expect(__builtin_amdgcn_ballot_w64(move) != 0, 0)) {
-            const float mx_abs = mx + m_ref;
-            const float new_run = ordinary ? mx_abs : fmaxf(m_run, mx_abs);
             // exp2(old reference - new reference); an unset reference (-inf) scales by 0
-            const float alpha = (m_run == -INFINITY) ? 0.f : fast_exp2(m_run - new_run);
+            const float alpha = (m_run == -INFINITY) ? 0.f : fast_exp2(m_run - mx);
             if (move) {
-                const float sub = ordinary ? mx : new_run - m_ref;
-                m_run = new_run;
-                m_ref = new_run > kHugeNeg ? new_run : 0.f;
+                m_run = mx;
+                m_ref = mx;
                 l_run *= alpha;
 #pragma unroll
                 for (int x = 0; x < DV; ++x)
 #pragma unroll
                     for (int r = 0; r < 16; ++r) o_acc[x][r] *= alpha;
-#pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    s0[r] -= sub;
-                    s1[r] -= sub;
-                    neg_m[r] = -m_ref;
-                }
             }
         }
     };
@@ -272,7 +255,7 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
     auto half_prob = [&](f32x16_t& s, int t, int kb, uint32_t (&pw)[8], uint32_t& drop_bits)
                          __attribute__((always_inline)) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) s[r] = fast_exp2(s[r]);
+        for (int r = 0; r < 16; ++r) s[r] = fast_exp2(s[r] - m_ref);
         if constexpr (kDrop != 0) {
             float psum = 0.f;
 #pragma unroll
@@ -338,7 +321,7 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
         half_scores(kt, 1, s1);
         const float mx =
             max_xor32(fmaxf(finish_half(s0, t, 0, mask_tag), finish_half(s1, t, 1, mask_tag)));
-        update_reference(mx, s0, s1);
+        update_reference(mx);
         uint32_t bits0 = 0, bits1 = 0;
         half_prob(s0, t, 0, pw0, bits0);
         half_accumulate(vt, 0, pw0);
@@ -440,20 +423,14 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
     // ---- epilogue ----
     const float l_tot = sum_xor32(l_run);
     const float inv_l = 1.0f / l_tot;
+    // every wavefront is past the last barrier of the loop: the K buffers are free, and each
+    // wavefront routes its 32 output rows through its own quarter of them
+    if (wq0 < a.sq) {
+        T* o_row0 = reinterpret_cast<T*>(a.o) + b * a.os[0] + (int64_t)wq0 * a.os[1] + h * a.os[2];
+        store_block_via_lds<T, DPAD, kPitch>(o_acc, inv_l, k_lds + wave * 32 * kPitch, o_row0,
+                                             a.os[1], a.sq - wq0, a.d);
+    }
     if (q_row < a.sq) {
-        T* o_row = reinterpret_cast<T*>(a.o) + b * a.os[0] + (int64_t)q_row * a.os[1] + h * a.os[2];
-#pragma unroll
-        for (int x = 0; x < DV; ++x)
-#pragma unroll
-            for (int r4 = 0; r4 < 4; ++r4) {
-                const int d0 = x * 32 + 8 * r4 + 4 * g;
-                if (d0 < a.d) {
-                    u32x2_t w;
-                    w.x = pack2<T>(o_acc[x][4 * r4 + 0] * inv_l, o_acc[x][4 * r4 + 1] * inv_l);
-                    w.y = pack2<T>(o_acc[x][4 * r4 + 2] * inv_l, o_acc[x][4 * r4 + 3] * inv_l);
-                    *reinterpret_cast<u32x2_t*>(o_row + d0) = w;
-                }
-            }
         // A row that met nothing but keys masked with a huge negative bias has a uniform softmax
         // here (as in the reference) but no log-sum-exp that fp32 can hold next to its scores:
         // +inf is stored, which makes the backward treat the row as contributing no gradient.
