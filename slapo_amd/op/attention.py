@@ -25,10 +25,12 @@ import logging
 from typing import Optional
 
 import torch
+import torch.nn.functional as F
 from torch import nn
 
 from ..random import draw_philox
 from . import _kernels as K
+from .fused_bias import bias_dropout
 
 logger = logging.getLogger("slapo_amd")
 
@@ -255,6 +257,15 @@ class FlashAttention(nn.Module):
         context_layer = context_layer.view(context_layer.size()[:-2] + (-1,))
 
         if self.output_proj:
-            context_layer = self.resid_dropout(self.out_proj(context_layer))
+            # out_proj's bias and resid_dropout ride on one pass over [B, S, hidden] (the reference
+            # runs the GEMM with bias, then nn.Dropout: slapo/op/attention.py:514-516).  The mask
+            # is the one nn.Dropout would draw; p and training are read from the child module, so
+            # schedules that edit `resid_dropout` keep working.
+            if self.out_proj.bias is not None:
+                context_layer = bias_dropout(
+                    F.linear(context_layer, self.out_proj.weight, None), self.out_proj.bias,
+                    self.resid_dropout.p, self.resid_dropout.training)
+            else:
+                context_layer = self.resid_dropout(self.out_proj(context_layer))
 
         return (context_layer, (key_layer, value_layer) if use_cache else None)

@@ -138,6 +138,14 @@ def draw_philox(offset_increment: int, device=None):
     Must be called from forward only; backward re-uses the pair saved in the autograd context."""
     if offset_increment % 4 != 0:
         raise ValueError("Philox offset increments are multiples of 4")
+    if torch.cuda.is_available() and torch.cuda.is_current_stream_capturing():
+        # The pair is read on the host and baked into the launch: a captured graph would replay
+        # one and the same mask.  Capture the C-ABI entry points with dropout off, or with
+        # caller-supplied (seed, offset) pairs, instead.
+        raise RuntimeError(
+            "slapo_amd: dropout with p > 0 draws (seed, offset) from the device generator on the "
+            "host and cannot be captured into a graph"
+        )
     gen = DeviceGeneratorBackend._gen(device)
     seed = gen.initial_seed()
     offset = gen.get_offset()
