@@ -242,6 +242,8 @@ def test_dropout_mask_bits_read_back_exactly():
     ((1, 320, 2, 128), True, 100, False, 0.1),  # local window (staggered variant at 128)
     ((1, 192, 2, 80), False, 0, True, 0.2),     # head_dim 80 (padded to 96)
     ((1, 320, 2, 80), True, 0, False, 0.1),     # ... causal: sequential and diagonal tile bodies
+    ((1, 1024, 8, 64), True, 0, False, 0.1),    # 8 Mi scores: four Philox loop trips per thread
+    ((1, 1024, 8, 128), False, 0, False, 0.2),  # ... without a mask, head_dim 128
 ])
 def test_dropout_keep_bits_saved_by_the_forward(dtype, shape, causal, window, masked, p):
     """The forward stores the keep bits, the backward reads them: gradients are bitwise those of
@@ -338,6 +340,52 @@ def test_argument_errors():
         op.hip_attention(odd, odd, odd)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+def test_attention_dropout_over_several_philox_trips(dtype):
+    """B 1, H 8, S 1024: 8 Mi scores are four loop trips of ATen's dropout launch (524 288 threads
+    x 4 elements), so the kernels' Philox counters run past their first value.  torch's own mask
+    (drawn for the dense fp32 [B*H, Sq, Sk] tensor), forward values and all three gradients
+    against the oracle evaluated with that mask."""
+    b, s, h, d, p = 1, 1024, 8, 64, 0.1
+    from slapo_amd.op import _kernels as K
+    plan = K.dropout_plan(b * h * s * s, 4, torch.device("cuda", 0))
+    assert b * h * s * s > plan.total_threads * 4  # more than one trip
+    q, k, v, do, _ = _inputs(b, s, h, d, dtype)
+    _check(q, k, v, do, None, True, 0, dtype, p=p)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("d,scale", [(80, 1.0), (128, 1.0), (128, 0.01), (64, 0.0), (80, -0.05)])
+def test_softmax_scale_other_than_the_default(dtype, d, scale):
+    """FlashAttentionOp(scale=...): GPT-Neo runs scale 1.0; a tiny, a zero (uniform attention)
+    and a negative scale are legal in the reference (slapo/op/attention.py:166-169) as well."""
+    q, k, v, do, _ = _inputs(2, 200, 2, d, dtype)
+    q = q * 0.3  # keep scale 1.0 scores in a range where 16-bit inputs still carry the answer
+    qd, kd, vd = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    out = op.FlashAttentionOp("hip_cdna4", apply_causal_mask=True, scale=scale)(qd, kd, vd, None, 0.0)
+    out.backward(do.cuda())
+    ro, rq, rk, rv = OA.attention_fwd_bwd(q, k, v, do, None, True, 0, 0.0, None, scale,
+                                          torch.float64)
+    for name, a, r in (("out", out, ro), ("dq", qd.grad, rq), ("dk", kd.grad, rk),
+                       ("dv", vd.grad, rv)):
+        assert_parity(a, r, dtype, name)
+
+
+# ---- the benchmark configurations at their full sequence length (batch / heads reduced) -------
+def test_cfg4_opt_at_seq_2048_against_the_oracle():
+    """bf16, S 2048, head_dim 80, causal + key padding (B 2, H 2; the fp64 oracle needs 270 MB)."""
+    q, k, v, do, g = _inputs(2, 2048, 2, 80, torch.bfloat16)
+    mask, _ = _padding_mask(2, 2048, torch.bfloat16, g, 512)
+    _check(q, k, v, do, mask, True, 0, torch.bfloat16)
+
+
+@pytest.mark.parametrize("window", [0, 256])
+def test_cfg5_gpt_neo_at_seq_2048_against_the_oracle(window):
+    """bf16, S 2048, head_dim 128, causal / window 256, dropout 0.1 (B 1, H 2)."""
+    q, k, v, do, _ = _inputs(1, 2048, 2, 128, torch.bfloat16)
+    _check(q, k, v, do, None, True, window, torch.bfloat16, p=0.1)
+
+
 # ---- full benchmark sizes through size-independent properties ---------------------------------
 def test_full_size_cfg2_properties():
     """fp16, B 8, S 1024, 16 x 64, causal, at full size: (1) V = const gives that const back
@@ -368,6 +416,100 @@ def test_full_size_cfg2_properties():
     a_ = (qh.grad.double() * q.double()).sum(dim=(1, 3))
     b_ = (kh.grad.double() * k.double()).sum(dim=(1, 3))
     assert ((a_ - b_).abs().max() / a_.abs().max()).item() <= 2e-2
+
+
+def _fp32_twin(q, k, v, do, mask, causal, window, p, seed):
+    """The library's independent fp32 FMA kernels on the same 16-bit values and the same seed."""
+    qf, kf, vf = (t.float().requires_grad_(True) for t in (q, k, v))
+    torch.cuda.manual_seed(seed)
+    ref = op.hip_attention(qf, kf, vf, mask, causal=causal, p=p, window=window)
+    ref.backward(do.float())
+    return ref, qf.grad, kf.grad, vf.grad
+
+
+def test_full_size_cfg4_properties():
+    """bf16, B 4, S 2048, 32 x 80, causal + key padding with valid lengths ~ U[512, 2048], at full
+    size: rows of P sum to one (V = 1 returns 1, also for queries in the padded region); query 0
+    returns V[0]; linearity in V; padded keys receive exactly zero dK, dV; agreement of all four
+    outputs with the fp32 FMA kernels run on the same bf16 values; sum_i dQ.q = sum_j dK.k."""
+    b, s, h, d = 4, 2048, 32, 80
+    g = torch.Generator().manual_seed(2013)
+    q, k, v, do = (torch.randn(b, s, h, d, generator=g).bfloat16().cuda() for _ in range(4))
+    mask, lens = _padding_mask(b, s, torch.bfloat16, g, 512)
+    mask = mask.cuda()
+    out1 = op.hip_attention(q, k, torch.ones_like(v), mask, causal=True)
+    assert (out1.float() - 1).abs().max().item() <= 1e-2
+    out = op.hip_attention(q, k, v, mask, causal=True)
+    assert torch.equal(out[:, 0], v[:, 0])
+    out2 = op.hip_attention(q, k, 2 * v, mask, causal=True)
+    assert rel_err(out2, 2 * out.double()) <= 1e-2
+    qh, kh, vh = (t.clone().requires_grad_(True) for t in (q, k, v))
+    op.hip_attention(qh, kh, vh, mask, causal=True).backward(do)
+    for bi in range(b):
+        n = int(lens[bi])
+        assert not kh.grad[bi, n:].any() and not vh.grad[bi, n:].any()
+        assert kh.grad[bi, :n].any()
+    ref, rq, rk, rv = _fp32_twin(q, k, v, do, mask, True, 0, 0.0, 1)
+    assert rel_err(out, ref) <= 2e-2
+    assert rel_err(qh.grad, rq) <= 2e-2
+    assert rel_err(kh.grad, rk) <= 2e-2
+    assert rel_err(vh.grad, rv) <= 2e-2
+    a_ = (qh.grad.double() * q.double()).sum(dim=(1, 3))
+    b_ = (kh.grad.double() * k.double()).sum(dim=(1, 3))
+    assert ((a_ - b_).abs().max() / a_.abs().max()).item() <= 2e-2
+
+
+@pytest.mark.parametrize("window", [0, 256])
+def test_full_size_cfg5_properties(window):
+    """bf16, B 4, S 2048, 16 x 128, causal (global and window 256), dropout 0.1, at full size
+    (268 M scores: 128 Philox loop trips).  The keep bits that the forward stores are torch's
+    mask for the dense fp32 [B*H, Sq, Sk] tensor wherever the forward visits; outputs and
+    gradients agree with the fp32 FMA kernels run under the same seed; with V = 1 every row
+    returns the kept share of its probabilities, which averages to 1 over a head."""
+    import ctypes
+
+    from slapo_amd.op import _kernels as K
+    from slapo_amd.op import attention as A
+
+    b, s, h, d, p = 4, 2048, 16, 128, 0.1
+    g = torch.Generator().manual_seed(2013)
+    q, k, v, do = (torch.randn(b, s, h, d, generator=g).bfloat16().cuda() for _ in range(4))
+    plan = K.dropout_plan(b * h * s * s, 4, q.device)
+    assert b * h * s * s >= 100 * plan.total_threads * 4
+    torch.cuda.manual_seed(5)
+    seed, offset = A.draw_philox(plan.offset_increment, q.device)
+    _, _, _, words = K.attn_fwd(q, k, v, None, True, window, d ** -0.5, p, seed, offset, plan,
+                                save_mask=True)
+    keep = _torch_keep(b, h, s, s, p).cuda()           # [bh, s, s] bool
+    n_words = s // 32
+    words = words.view(b * h, n_words, s).to(torch.int64) & 0xFFFFFFFF
+    i = torch.arange(s, device="cuda")
+    # compare word by word: pack torch's mask the same way
+    weights = (1 << torch.arange(32, device="cuda", dtype=torch.int64))
+    packed = (keep.view(b * h, s, n_words, 32).to(torch.int64) * weights).sum(-1)  # [bh, i, w]
+    packed = packed.permute(0, 2, 1)                                                # [bh, w, i]
+    w = torch.arange(n_words, device="cuda")
+    # a 32-key word is written iff its 64-key tile is visited by the 32-query group of the row
+    tile0 = (w[:, None] // 2) * 64
+    grp0 = (i[None, :] // 32) * 32
+    visited = tile0 <= grp0 + 31
+    if window:
+        visited &= grp0 - (tile0 + 63) < window
+    assert torch.equal(words[:, visited], packed[:, visited])
+    del keep, packed, words
+
+    torch.cuda.manual_seed(9)
+    out1 = op.hip_attention(q, k, torch.ones_like(v), None, causal=True, p=p, window=window)
+    assert abs(out1.float().mean().item() - 1.0) <= 5e-3
+    qh, kh, vh = (t.clone().requires_grad_(True) for t in (q, k, v))
+    torch.cuda.manual_seed(9)
+    out = op.hip_attention(qh, kh, vh, None, causal=True, p=p, window=window)
+    out.backward(do)
+    ref, rq, rk, rv = _fp32_twin(q, k, v, do, None, True, window, p, 9)
+    assert rel_err(out, ref) <= 2e-2
+    assert rel_err(qh.grad, rq) <= 2e-2
+    assert rel_err(kh.grad, rk) <= 2e-2
+    assert rel_err(vh.grad, rv) <= 2e-2
 
 
 def test_backward_is_bitwise_reproducible_and_stages_compose():
