@@ -15,8 +15,16 @@ epilogue  GB/s of the two FusedMLP epilogues (bf16, tokens 8192, 1024 -> 4096 ->
           HBM peak, on a rotating working set larger than the caches
 other_attention  forward and backward time of the OPT-2.7B-shaped (padding mask) and the two
           GPT-Neo-1.3B-shaped (global / window 256, dropout 0.1) attention calls, bf16
+bert_large_fp32  BASELINE configuration 1, which is DEFINED as the native CPU path: the oracle's
+          fp32 forward of B 4, S 512, 16 x 64 on the host cores, and beside it the fp32 FMA kernel
+          of this library on the same tensors against the fp32 vector peak (reported, not a target)
 cpu_baseline  the oracle's native-PyTorch restatement (fp32 CPU, autograd backward) timed on the
-          host cores on a bounded sample of the same workload
+          host cores on a bounded sample of the same workload; every epilogue / other_attention
+          entry carries a cpu_baseline of its own (a bounded chunk of its tensors)
+
+The headline is the MEDIAN of `--repeats` (default 5) timed loops of `--steps` steps each, every
+loop bracketed by a device synchronisation on both sides; `ms_per_step` x `steps` is the duration
+of that median loop.
 """
 from __future__ import annotations
 
@@ -34,6 +42,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 MFMA_PEAK_TFLOPS = 2500.0  # MI355X dense fp16 / bf16
+FP32_VECTOR_PEAK_TFLOPS = 157.3
 # HBM bytes per launch of the dK/dV kernel on WORKLOAD, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE (KiB per dispatch), each scaled by the same counter's reading for a 256 MiB copy
 # (FETCH_SIZE reads half the copied bytes: factor 2.0; WRITE_SIZE factor 1.0):
@@ -250,12 +259,156 @@ def bench_epilogues(device, iters=40):
     return out
 
 
+def _cpu_info():
+    """Host description that goes with every CPU figure: logical cores, threads used, model."""
+    model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    return {"os_cpu_count": os.cpu_count(), "torch_num_threads": torch.get_num_threads(),
+            "cpu_model": model}
+
+
+def _use_all_cores():
+    torch.set_num_threads(os.cpu_count() or 1)
+    return torch.get_num_threads()
+
+
+def _median_time(fn, reps=3):
+    fn()  # warm-up
+    times = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - t0)
+    return sorted(times)[len(times) // 2]
+
+
+def cpu_epilogue_baselines():
+    """The oracle's epilogues and cross entropy (native PyTorch, fp32 math on 16-bit values) on
+    4096 of the 8192 rows (cross entropy: 512); GB/s count the same algorithmic bytes per row as
+    the GPU entries."""
+    from oracle import cross_entropy as OC
+    from oracle import epilogue as OE
+
+    threads = _use_all_cores()
+    rows, T, I, Hd, e = 4096, 8192, 4096, 1024, 2
+    g = torch.Generator().manual_seed(2013)
+    bf = torch.bfloat16
+    y = torch.randn(rows, I, generator=g).to(bf)
+    bi = torch.randn(I, generator=g).to(bf)
+    gr = torch.randn(rows, I, generator=g).to(bf)
+    x = torch.randn(rows, Hd, generator=g).to(bf)
+    b1 = torch.randn(Hd, generator=g).to(bf)
+    res = torch.randn(rows, Hd, generator=g).to(bf)
+    keep = torch.rand(rows, Hd, generator=g) >= 0.1
+    w, lb = torch.ones(Hd), torch.zeros(Hd)
+    sample = f"{rows} of {T} rows, fp32 math, median of 3"
+    out = {}
+
+    def entry(name, nbytes_full, fn):
+        sec = _median_time(fn)
+        out[name] = {"value": nbytes_full * rows / T / sec / 1e9, "unit": "GB/s", "cores": threads,
+                     "kind": "port", "sample": f"{sample}, {sec * 1e3:.1f} ms per pass"}
+
+    entry("bias_gelu_fwd", 2 * T * I * e + I * e,
+          lambda: OE.bias_gelu(bi, y, torch.float32).to(bf))
+    entry("bias_gelu_bwd", 3 * T * I * e + 2 * I * e,
+          lambda: OE.bias_gelu_back(gr, bi, y, torch.float32).to(bf))
+    entry("bias_dropout_residual_fwd", 3 * T * Hd * e + Hd * e,
+          lambda: OE.bias_dropout_residual(x, b1, res, 0.1, keep, torch.float32).to(bf))
+    entry("bias_dropout_residual_ln_fwd", 4 * T * Hd * e + 3 * Hd * e + 2 * T * 4,
+          lambda: OE.bias_dropout_residual_layer_norm(x, b1, res, w, lb, 1e-5, 0.1, keep,
+                                                      torch.float32)[0].to(bf))
+    _, z, mean, rstd = OE.bias_dropout_residual_layer_norm(x, b1, res, w, lb, 1e-5, 0.1, keep,
+                                                           torch.float32, z_dtype=bf)
+    gy = torch.randn(rows, Hd, generator=g).to(bf)
+    entry("bias_dropout_residual_ln_bwd", 4 * T * Hd * e + 4 * Hd * e + 2 * T * 4,
+          lambda: OE.bias_dropout_residual_layer_norm_bwd(gy, z, mean, rstd, w, 0.1, keep,
+                                                          torch.float32)[0].to(bf))
+    rows_ce, V = 512, 50257
+    logits = torch.randn(rows_ce, V, generator=g).to(torch.float16)
+    tgt = torch.randint(0, V, (rows_ce,), generator=g)
+    ones = torch.ones(rows_ce)
+    rows = rows_ce
+    sample = f"{rows} of {T} rows, fp32 math, median of 3"
+    entry("vocab_ce_fwd", T * V * 2 + T * (8 + 16),
+          lambda: OC.forward(logits, tgt, 0.0, torch.float32)[0])
+    soft = OC.forward(logits, tgt, 0.0, torch.float32)[1]
+    entry("vocab_ce_bwd", 2 * T * V * 2 + T * (8 + 12),
+          lambda: OC.backward(soft, tgt, ones).to(torch.float16))
+    return out
+
+
+def cpu_attention_chunk(cfg, heads, lens=None):
+    """The oracle's attention fwd+bwd (fp32 CPU, autograd) on one batch and `heads` heads of an
+    other_attention workload; TFLOP/s count 14 * D per attended pair of the chunk."""
+    from oracle import attention as OA
+
+    threads = _use_all_cores()
+    S, D, w, p = cfg["seq"], cfg["head_dim"], cfg["window"], cfg["p"]
+    g = torch.Generator().manual_seed(2013)
+    q, k, v, do = (torch.randn((1, S, heads, D), generator=g).to(torch.bfloat16) for _ in range(4))
+    mask, n = None, S
+    if lens is not None:
+        n = lens[0]
+        mask = torch.zeros(1, 1, 1, S)
+        mask[0, 0, 0, n:] = torch.finfo(torch.bfloat16).min
+    keep = (torch.rand(heads, S, S, generator=g) >= p) if p > 0 else None
+    sec = _median_time(lambda: OA.attention_fwd_bwd(q, k, v, do, mask, True, w, p, keep, None,
+                                                    torch.float32), reps=3)
+    pairs = OA.attended_pairs(S, S, True, w, n) * heads
+    return {"value": 14 * D * pairs / sec / 1e12, "unit": "TFLOP/s", "cores": threads,
+            "kind": "port", "sample": f"1 of {cfg['batch']} batches, {heads} of {cfg['heads']} "
+                                      f"heads, fp32 math on bf16 inputs, {sec:.2f} s per pass"}
+
+
+def bench_bert_large_fp32(device, iters=10):
+    """BASELINE configuration 1: BERT-large-shaped self-attention, fp32, B 4, S 512, 16 x 64, no
+    mask, dropout 0, forward only.  The configuration is defined as the native CPU path, so the
+    CPU time of the oracle IS its figure; the library's fp32 FMA kernel runs beside it."""
+    from oracle import attention as OA
+    from slapo_amd import op
+
+    threads = _use_all_cores()
+    B, S, H, D = 4, 512, 16, 64
+    g = torch.Generator().manual_seed(2013)
+    q, k, v = (torch.randn((B, S, H, D), generator=g) for _ in range(3))
+    flops = 4 * D * S * S * B * H
+    cpu_sec = _median_time(lambda: OA.xformers_ref(q, k, v, None, False,
+                                                   compute_dtype=torch.float32))
+    qd, kd, vd = (t.to(device) for t in (q, k, v))
+    for _ in range(3):
+        op.hip_attention(qd, kd, vd, None, causal=False)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(iters):
+        op.hip_attention(qd, kd, vd, None, causal=False)
+    e1.record()
+    torch.cuda.synchronize()
+    gpu_sec = e0.elapsed_time(e1) / iters * 1e-3
+    return {"workload": "bert-large self-attention forward, fp32, B4 S512 H16 D64, no mask",
+            "flops": flops,
+            "cpu": {"ms": cpu_sec * 1e3, "TFLOPs": flops / cpu_sec / 1e12, "cores": threads,
+                    "kind": "port", "sample": "the whole configuration, median of 3"},
+            "gpu_fp32_fma_kernel": {"ms": gpu_sec * 1e3, "TFLOPs": flops / gpu_sec / 1e12,
+                                    "peak": FP32_VECTOR_PEAK_TFLOPS,
+                                    "frac_of_fp32_vector_peak":
+                                        flops / gpu_sec / 1e12 / FP32_VECTOR_PEAK_TFLOPS,
+                                    "note": "parity kernel (1e-5 bar), not a performance target"}}
+
+
 def cpu_baseline(cfg, budget_batches=8):
     """The oracle's native path (fp32 CPU, autograd) on `budget_batches` of the 8 batches."""
     from oracle import attention as OA
 
-    threads = min(os.cpu_count() or 1, 16)
-    torch.set_num_threads(threads)
+    threads = _use_all_cores()
     g = torch.Generator().manual_seed(cfg["seed"])
     shape = (budget_batches, cfg["seq"], cfg["heads"], cfg["head_dim"])
     q, k, v, do = (torch.randn(shape, generator=g).to(torch.float16) for _ in range(4))
@@ -266,12 +419,12 @@ def cpu_baseline(cfg, budget_batches=8):
         return time.perf_counter() - t0
 
     run()  # warm-up
-    times = sorted(run() for _ in range(3))
-    sec = times[1]
+    times = sorted(run() for _ in range(9))
+    sec = times[4]
     flops = 14 * cfg["head_dim"] * _pairs(cfg["seq"], cfg["causal"]) * budget_batches * cfg["heads"]
     return {"value": flops / sec / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
             "sample": f"{budget_batches} of {cfg['batch']} batches of the same workload "
-                      f"(fp32 math on fp16 inputs, median of 3, {sec:.2f} s per pass)"}
+                      f"(fp32 math on fp16 inputs, median of 9, {sec:.2f} s per pass)"}
 
 
 OTHER_ATTENTION = [
@@ -284,7 +437,7 @@ OTHER_ATTENTION = [
 ]
 
 
-def bench_other_attention(device, iters=20):
+def bench_other_attention(device, iters=20, with_cpu=True):
     """Forward and backward time of the other attention shapes of the benchmark set (bf16), through
     the C ABI on preallocated buffers; TFLOP/s count 14 * D FLOP per attended (query, key) pair.
     The padding mask is the compact additive [B,1,1,Sk] tensor with per-sequence valid lengths
@@ -350,11 +503,23 @@ def bench_other_attention(device, iters=20):
             return e0.elapsed_time(e1) / iters * 1e-3
 
         tf, tb = timed(fwd), timed(bwd)
+        stage_us = {}
+        for name, bits in (("dq_us", _lib.BWD_PREPARE | _lib.BWD_DQ), ("dkdv_us", _lib.BWD_DKDV)):
+            def one(bits=bits):
+                rc = lib.slapo_amd_attn_bwd_stages(ctypes.byref(prm), P(q), P(k), P(v), P(bias),
+                                                   P(o), P(do), P(lse), P(dq), P(dk), P(dv),
+                                                   *strides, P(ws), nbytes, bits, st)
+                if rc:
+                    raise RuntimeError(f"slapo_amd_attn_bwd_stages failed with status {rc}")
+            stage_us[name] = timed(one) * 1e6
         tflops = 14 * D * pairs / (tf + tb) / 1e12
-        out.append({"workload": cfg["name"], "dtype": "bf16", "batch": B, "seq_len": S, "heads": H,
-                    "head_dim": D, "window": w, "dropout_p": cfg["p"], "attended_pairs": pairs,
-                    "fwd_us": tf * 1e6, "bwd_us": tb * 1e6, "TFLOPs": tflops,
-                    "frac_of_mfma_peak": tflops / MFMA_PEAK_TFLOPS})
+        entry = {"workload": cfg["name"], "dtype": "bf16", "batch": B, "seq_len": S, "heads": H,
+                 "head_dim": D, "window": w, "dropout_p": cfg["p"], "attended_pairs": pairs,
+                 "fwd_us": tf * 1e6, "bwd_us": tb * 1e6, **stage_us, "TFLOPs": tflops,
+                 "frac_of_mfma_peak": tflops / MFMA_PEAK_TFLOPS}
+        if with_cpu:
+            entry["cpu_baseline"] = cpu_attention_chunk(cfg, 16, lens if cfg["padding"] else None)
+        out.append(entry)
         del q, k, v, do, o, lse, dq, dk, dv, ws, keep, bias
     return out
 
@@ -364,6 +529,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--repeats", type=int, default=5,
+                    help="timed loops of --steps steps; the median loop is reported")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-epilogues", action="store_true")
     ap.add_argument("--no-other-attention", action="store_true",
@@ -399,17 +566,24 @@ def main():
     every = 4
     events = [[torch.cuda.Event(enable_timing=True) for _ in range(4)]
               for _ in range((args.steps + every - 1) // every)]
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        step.step(events[i // every] if i % every == 0 else None)
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
+    loops = []
+    for _ in range(max(1, args.repeats)):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(args.steps):
+            step.step(events[i // every] if i % every == 0 else None)
+        torch.cuda.synchronize()
+        loops.append(time.perf_counter() - t0)
+        torch.cuda.synchronize()
+        seg = [sum(ev[i].elapsed_time(ev[i + 1]) for ev in events) / len(events) for i in range(3)]
+        loops[-1] = (loops[-1], seg)
+    loops.sort(key=lambda t: t[0])
+    elapsed, seg_ms = loops[len(loops) // 2]
 
     n_pairs = _pairs(cfg["seq"], cfg["causal"]) * cfg["batch"] * cfg["heads"]
     d = cfg["head_dim"]
     ms_per_step = elapsed / args.steps * 1e3
     value = 14 * d * n_pairs / (elapsed / args.steps) / 1e12
-    seg_ms = [sum(ev[i].elapsed_time(ev[i + 1]) for ev in events) / len(events) for i in range(3)]
     kern_ms = seg_ms[2]
     bwd_flops = 8 * d * n_pairs
     achieved = bwd_flops / (kern_ms * 1e-3) / 1e12
@@ -426,7 +600,9 @@ def main():
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "repeats": len(loops),
         "ms_per_step": ms_per_step,
+        "ms_per_step_of_every_loop": [t / args.steps * 1e3 for t, _ in loops],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -445,12 +621,18 @@ def main():
     result["kernels"] = [kern("attn_fwd_kernel<f16,64,0,0,0>", 4 * d * n_pairs, seg_ms[0]),
                          kern("attn_bwd_kernel<f16,64,0,0,1> (dK/dV)", bwd_flops, seg_ms[2]),
                          kern("attn_bwd_dq_kernel<f16,64,0,0,true>", 6 * d * n_pairs, seg_ms[1])]
+    with_cpu = not args.no_cpu_baseline
     if not args.no_epilogues:
         result["epilogue"] = bench_epilogues(device)
+        if with_cpu:
+            for name, base in cpu_epilogue_baselines().items():
+                result["epilogue"][name]["cpu_baseline"] = base
     if not args.no_other_attention:
-        result["other_attention"] = bench_other_attention(device)
-    if not args.no_cpu_baseline:
+        result["other_attention"] = bench_other_attention(device, with_cpu=with_cpu)
+    if with_cpu:
+        result["bert_large_fp32"] = bench_bert_large_fp32(device)
         result["cpu_baseline"] = cpu_baseline(cfg)
+        result["host"] = _cpu_info()
     print(json.dumps(result))
 
 
