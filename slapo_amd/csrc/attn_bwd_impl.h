@@ -325,19 +325,10 @@ __global__ __launch_bounds__(kBwdThreads, (bwd_two_per_cu(DPAD, kDrop, KB) ? 2 :
         }
     };
     // Keep-bits of one key block of a half tile: wq[e] bit 4 * r4 belongs to register 4 * r4 + e.
-    // mask_h (kDrop == 3): the words of this wavefront's keys for the 32 queries of the half
-    auto keep_bits_half = [&](int kcol, int ih0, const uint32_t* mask_h, uint32_t (&wq)[4])
+    // (kDrop == 3 reads the stored words in half_ds instead.)
+    auto keep_bits_half = [&](int kcol, int ih0, uint32_t (&wq)[4])
                               __attribute__((always_inline)) {
-        if constexpr (kDrop == 3) {
-#pragma unroll
-            for (int r4 = 0; r4 < 4; ++r4) {
-                const u32x4_t w = *reinterpret_cast<const u32x4_t*>(mask_h + quad_slot(r4, g));
-                wq[0] |= ((w.x >> c_loc) & 1u) << (4 * r4);
-                wq[1] |= ((w.y >> c_loc) & 1u) << (4 * r4);
-                wq[2] |= ((w.z >> c_loc) & 1u) << (4 * r4);
-                wq[3] |= ((w.w >> c_loc) & 1u) << (4 * r4);
-            }
-        } else if constexpr (kDrop == 1) {
+        if constexpr (kDrop == 1) {
             // The four lanes of a quad hold four consecutive keys, i.e. one Philox block per query
             // row.  Lane j of the quad draws the blocks of the rows held in registers j, j+4, j+8,
             // j+12 and the quad exchanges them: 4 blocks per lane instead of 16.
@@ -380,25 +371,32 @@ __global__ __launch_bounds__(kBwdThreads, (bwd_two_per_cu(DPAD, kDrop, KB) ? 2 :
         for (int kb = 0; kb < KB; ++kb) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) wq[kb][e] = 0u;
-            keep_bits_half(key[kb], ih0, mask_h, wq[kb]);
+            keep_bits_half(key[kb], ih0, wq[kb]);
         }
 #pragma unroll
         for (int r4 = 0; r4 < 4; ++r4) {
             f32x4_t del4 = {0.f, 0.f, 0.f, 0.f};  // no dropout: already subtracted
+            u32x4_t w4 = {0u, 0u, 0u, 0u};
             if constexpr (kDrop != 0)
                 del4 = *reinterpret_cast<const f32x4_t*>(delta_h + quad_slot(r4, g));
+            // kDrop == 3: the stored words of four queries (bit j = key j of this wavefront)
+            if constexpr (kDrop == 3)
+                w4 = *reinterpret_cast<const u32x4_t*>(mask_h + quad_slot(r4, g));
 #pragma unroll
             for (int kb = 0; kb < KB; ++kb) {
                 float pv[4], dv[4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    float pe = p[kb][4 * r4 + e];
+                    const float pe = p[kb][4 * r4 + e];
                     float d = dp[kb][4 * r4 + e];
                     float pd = pe;
                     if constexpr (kDrop != 0) {
-                        const float keep = ((wq[kb][e] >> (4 * r4)) & 1u) ? a.rng.inv_keep : 0.f;
-                        pd = pe * keep;
-                        d = d * keep;
+                        // dropped pairs become +0; dV takes its factor 1 / (1 - p) when it is
+                        // written, dP takes it here
+                        const uint32_t bits = kDrop == 3 ? w4[e] : wq[kb][e];
+                        const uint32_t pos = kDrop == 3 ? (uint32_t)c_loc : 4u * r4;
+                        pd = keep_or_zero(pe, bits, pos);
+                        d = keep_or_zero(d, bits, pos) * a.rng.inv_keep;
                     }
                     pv[e] = pd;
                     dv[e] = pe * (d - del4[e]);
@@ -581,8 +579,10 @@ __global__ __launch_bounds__(kBwdThreads, (bwd_two_per_cu(DPAD, kDrop, KB) ? 2 :
             reinterpret_cast<T*>(a.dv) + b * a.dvs[0] + (int64_t)kw0 * a.dvs[1] + h * a.dvs[2];
         store_block_via_lds<T, DPAD, kPitch>(dk_acc[0], a.scale, q_lds + wave * 32 * kPitch,
                                              dk_row0, a.dks[1], a.sk - kw0, a.d);
-        store_block_via_lds<T, DPAD, kPitch>(dv_acc[0], 1.0f, g_lds + wave * 32 * kPitch, dv_row0,
-                                             a.dvs[1], a.sk - kw0, a.d);
+        // with dropout: the factor 1 / (1 - p) that half_ds left out of P
+        store_block_via_lds<T, DPAD, kPitch>(dv_acc[0], kDrop != 0 ? a.rng.inv_keep : 1.0f,
+                                             g_lds + wave * 32 * kPitch, dv_row0, a.dvs[1],
+                                             a.sk - kw0, a.d);
     }
 }
 

@@ -185,6 +185,14 @@ __device__ __forceinline__ u32x4_t keep_or_zero(u32x4_t v, bool keep) {
     return u32x4_t{v.x & m, v.y & m, v.z & m, v.w & m};
 }
 
+// v where bit `pos` of `bits` is set, +0 elsewhere: the bit, sign-extended to a whole word
+// (v_bfe_i32), masks the float.  Two instructions per value where a test, a compare and a select
+// take three.
+__device__ __forceinline__ float keep_or_zero(float v, uint32_t bits, uint32_t pos) {
+    const uint32_t m = (uint32_t)__builtin_amdgcn_sbfe((int)bits, pos, 1u);
+    return __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, v) & m);
+}
+
 // Kernel argument block (filled by the host dispatcher from slapo_attn_params).
 struct AttnArgs {
     const void* q;
@@ -205,9 +213,9 @@ struct AttnArgs {
     int has_bias, bias_vec4;  // bias_vec4: s3 == 1, s2 == 0 rows 16B-aligned
     // dropout: 0 = off, 1 = fast mask geometry (plan.vec >= 4, power-of-two thread count and
     // sk % 4 == 0: one Philox block per aligned group of four keys), 2 = any geometry,
-    // 3 (backward only) = keep bits read from keep_mask
+    // 3 = keep bits read from keep_mask (drawn by keep_mask_kernel ahead of the forward)
     int dropout;
-    // Keep bits of the dropout mask, written by the forward when not null: uint32 words
+    // Keep bits of the dropout mask, when not null: uint32 words
     // [batch*heads][mask_words][mask_pitch], bit j of word (bh, w, i) = keep(query i, key 32 w + j)
     uint32_t* keep_mask;
     int mask_words, mask_pitch;

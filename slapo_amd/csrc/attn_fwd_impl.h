@@ -252,8 +252,30 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
             }
         }
     };
+    // Keep bits of this lane's query for the 32 keys from j0 on (bit j = key j0 + j), drawn here:
+    // Philox blocks cover four consecutive keys; the two lanes of a query (l, l ^ 32) draw the
+    // blocks of keys 8 g .. 8 g + 7 of each 16-key group and exchange them.
+    auto draw_half = [&](int j0) __attribute__((always_inline)) -> uint32_t {
+        uint32_t mine = 0;
+#pragma unroll
+        for (int blk = 0; blk < 4; ++blk) {
+            const int pos = 16 * (blk >> 1) + 8 * g + 4 * (blk & 1);
+            const int key0 = j0 + pos;
+            uint32_t bits = 0;
+            if (q_row < a.sq && key0 < a.sk) {
+                const uint64_t e0 = drop_row_base + (uint64_t)key0;
+                if constexpr (kDrop == 1)
+                    bits = dropout_keep4_pow2(a.rng, e0 >> 2);
+                else
+                    bits = dropout_keep_any(a.rng, e0, min(4, a.sk - key0));
+            }
+            mine |= bits << pos;
+        }
+        return or_xor32(mine);
+    };
     // probabilities of one half: exp2, dropout, pack to T, row sum
-    // (drop_bits: the keep bits of this lane's 16 keys at their position in the half)
+    // (drop_bits: the keep bits of this lane's query for the 32 keys of the half; kDrop == 3
+    // passes in the word that keep_mask_kernel stored, the other modes return the drawn one)
     auto half_prob = [&](f32x16_t& s, int t, int kb, uint32_t (&pw)[8], uint32_t& drop_bits)
                          __attribute__((always_inline)) {
 #pragma unroll
@@ -263,26 +285,8 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
 #pragma unroll
             for (int r = 0; r < 16; ++r) psum += s[r];
             l_run += psum;
-            // Philox blocks cover four consecutive keys; the two lanes of a query (l, l ^ 32)
-            // draw the blocks of keys 8 g .. 8 g + 7 of each 16-key group and exchange them.  The
-            // combined word (bit j = key j of the half) is also what the backward reads.
-            const int j0 = t * kBN + 32 * kb;
-            uint32_t mine = 0;
-#pragma unroll
-            for (int blk = 0; blk < 4; ++blk) {
-                const int pos = 16 * (blk >> 1) + 8 * g + 4 * (blk & 1);
-                const int key0 = j0 + pos;
-                uint32_t bits = 0;
-                if (q_row < a.sq && key0 < a.sk) {
-                    const uint64_t e0 = drop_row_base + (uint64_t)key0;
-                    if constexpr (kDrop == 1)
-                        bits = dropout_keep4_pow2(a.rng, e0 >> 2);
-                    else
-                        bits = dropout_keep_any(a.rng, e0, min(4, a.sk - key0));
-                }
-                mine |= bits << pos;
-            }
-            mine = or_xor32(mine);
+            uint32_t mine = drop_bits;
+            if constexpr (kDrop != 3) mine = draw_half(t * kBN + 32 * kb);
             const uint32_t mine_g = mine >> (kAccGroupStep * g);
 #pragma unroll
             for (int r = 0; r < 16; ++r)
@@ -319,12 +323,21 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
                          __attribute__((always_inline)) {
         f32x16_t s0, s1;
         uint32_t pw0[8], pw1[8];
+        uint32_t bits0 = 0, bits1 = 0;
+        if constexpr (kDrop == 3) {
+            // the keep bits of this lane's query for the two halves of the tile, drawn by
+            // keep_mask_kernel; requested first, used after the scores
+            const int w = 2 * t;
+            const int64_t base = (int64_t)bh * a.mask_words;
+            const int row = min(q_row, a.sq - 1);
+            bits0 = a.keep_mask[(base + min(w, a.mask_words - 1)) * a.mask_pitch + row];
+            bits1 = a.keep_mask[(base + min(w + 1, a.mask_words - 1)) * a.mask_pitch + row];
+        }
         half_scores(kt, 0, s0);
         half_scores(kt, 1, s1);
         const float mx =
             max_xor32(fmaxf(finish_half(s0, t, 0, mask_tag), finish_half(s1, t, 1, mask_tag)));
         update_reference(mx);
-        uint32_t bits0 = 0, bits1 = 0;
         half_prob(s0, t, 0, pw0, bits0);
         half_accumulate(vt, 0, pw0);
         half_prob(s1, t, 1, pw1, bits1);
@@ -333,7 +346,7 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
         // The (wavefront-uniform) branch sits at the end of the tile, where the basic block ends
         // anyway; inside the body it would keep the scheduler from mixing the Philox arithmetic
         // with the matrix instructions (10 % of the forward).
-        if constexpr (kDrop != 0) {
+        if constexpr (kDrop == 1 || kDrop == 2) {
             if (a.keep_mask != nullptr) {
                 const uint32_t w0 = bits0, w1 = bits1;  // already combined over the lane pair
                 uint32_t* row = a.keep_mask +
@@ -465,6 +478,9 @@ template <typename T, int DPAD, int kWin>
 int dispatch_nobias(const AttnArgs& a, hipStream_t st) {
     if (a.dropout == 1) return launch<T, DPAD, 0, 1, kWin>(a, st);
     if (a.dropout == 2) return launch<T, DPAD, 0, 2, kWin>(a, st);
+    if constexpr (kWin != 0) {  // stored keep bits: local-window calls only, see attn_capi.hip
+        if (a.dropout == 3) return launch<T, DPAD, 0, 3, kWin>(a, st);
+    }
     return launch<T, DPAD, 0, 0, kWin>(a, st);
 }
 template <typename T, int DPAD>
@@ -475,11 +491,13 @@ int dispatch_flags(const AttnArgs& a, hipStream_t st) {
         if (a.bs[2] == 0) {  // the bias depends on the key only
             if (a.dropout == 1) return launch<T, DPAD, 2, 1, 2>(a, st);
             if (a.dropout == 2) return launch<T, DPAD, 2, 2, 2>(a, st);
+            if (a.dropout == 3) return launch<T, DPAD, 2, 3, 2>(a, st);
             if (a.window <= 0) return launch<T, DPAD, 2, 0, 0>(a, st);
             return launch<T, DPAD, 2, 0, 2>(a, st);
         }
         if (a.dropout == 1) return launch<T, DPAD, 1, 1, 2>(a, st);
         if (a.dropout == 2) return launch<T, DPAD, 1, 2, 2>(a, st);
+        if (a.dropout == 3) return launch<T, DPAD, 1, 3, 2>(a, st);
         return launch<T, DPAD, 1, 0, 2>(a, st);
     }
     return a.window > 0 ? dispatch_nobias<T, DPAD, 1>(a, st) : dispatch_nobias<T, DPAD, 0>(a, st);

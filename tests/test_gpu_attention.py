@@ -239,7 +239,9 @@ def test_dropout_mask_bits_read_back_exactly():
     ((1, 200, 3, 64), False, 0, True, 0.3),     # ragged tail, padding mask (skipped key tiles)
     ((1, 131, 2, 32), True, 0, False, 0.5),     # Sk % 4 != 0: per-element mask geometry
     ((1, 320, 2, 128), True, 0, False, 0.1),    # sequential halves, two workgroups per CU
-    ((1, 320, 2, 128), True, 100, False, 0.1),  # local window (staggered variant at 128)
+    ((1, 320, 2, 128), True, 100, False, 0.1),  # local window: keep bits drawn ahead of the forward
+    ((2, 330, 2, 64), True, 70, True, 0.2),     # ... with a padding mask and a ragged tail
+    ((1, 203, 2, 80), True, 48, False, 0.3),    # ... Sk % 4 != 0: per-element mask geometry
     ((1, 192, 2, 80), False, 0, True, 0.2),     # head_dim 80 (padded to 96)
     ((1, 320, 2, 80), True, 0, False, 0.1),     # ... causal: sequential and diagonal tile bodies
     ((1, 1024, 8, 64), True, 0, False, 0.1),    # 8 Mi scores: four Philox loop trips per thread
