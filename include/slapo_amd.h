@@ -219,10 +219,12 @@ typedef struct slapo_attn_params {
      * probability tensor (only read when p_drop > 0) */
     slapo_dropout_plan plan;
     /* Optional (may be NULL), 16-bit types with p_drop > 0 only: device buffer of
-     * slapo_amd_attn_keep_mask_bytes(prm) bytes.  The forward stores the dropout keep bits in it
-     * (one bit per score), and a backward that is given the same buffer reads them instead of
-     * drawing every Philox block again in both of its kernels.  The results are bitwise the
-     * same with and without it.  Layout: uint32 words [batch*heads][ceil(seqlen_k/32)][pitch],
+     * slapo_amd_attn_keep_mask_bytes(prm) bytes.  The forward call stores the dropout keep bits
+     * in it (one bit per score; with window > 0 a kernel launched ahead of the forward kernel on
+     * the same stream draws them and the forward kernel reads them), and a backward that is given
+     * the same buffer reads them instead of drawing every Philox block again in both of its
+     * kernels.  The results are bitwise the same with and without it.  Words whose keys no query
+     * of the row's 32-query group can see under the causal mask or the window are not written.  Layout: uint32 words [batch*heads][ceil(seqlen_k/32)][pitch],
      * pitch = seqlen_q rounded up to 4; bit j of word (bh, w, i) = keep(query i, key 32 w + j). */
     void* keep_mask;
 } slapo_attn_params;
