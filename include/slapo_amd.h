@@ -232,7 +232,11 @@ typedef struct slapo_attn_params {
 /* Size in bytes of the keep_mask buffer (0 when p_drop == 0 or the type is SLAPO_F32). */
 size_t slapo_amd_attn_keep_mask_bytes(const slapo_attn_params* prm);
 
-/* lse: [batch, heads, seqlen_q] fp32, natural-log sum-exp of the masked, scaled scores. */
+/* lse: [batch, heads, seqlen_q] fp32, natural-log sum-exp of the masked, scaled scores.  Bias
+ * values at or below -5e8 (other than -inf) are one masking value; a query row that sees nothing
+ * but keys masked with it attends to them uniformly, as in the reference's arithmetic, and its
+ * lse slot holds n * 2^100 (n = number of those keys) for the backward, which gives such rows the
+ * gradients of that uniform softmax. */
 int slapo_amd_attn_fwd(const slapo_attn_params* prm, const void* q, const void* k, const void* v,
                        const float* bias, void* o, float* lse, void* stream);
 

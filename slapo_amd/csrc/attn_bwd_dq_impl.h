@@ -117,7 +117,7 @@ __global__ __launch_bounds__(kThreads, (kStagger && DPAD > 64 ? 1 : 2)) void att
     const int n_tiles = t_hi - t_lo;
 
     frag_t qf[DK], gf[DK];
-    float lse2, delta;
+    float lse2, delta, inv_n = 1.0f;
     {
         const int qr = min(q_row, a.sq - 1);
         const T* o_base = reinterpret_cast<const T*>(a.o) + b * a.os[0] + h * a.os[2];
@@ -143,8 +143,13 @@ __global__ __launch_bounds__(kThreads, (kStagger && DPAD > 64 ? 1 : 2)) void att
         for (int t = 0; t < DK; ++t) {
             qf[t] = scale_frag<T>(__builtin_bit_cast(u32x4_t, qf[t]), a.scale_log2);
         }
-        // log2 units; +inf for rows past the end so that P = 0 there
-        lse2 = row_ok ? lse_raw * kLog2e : INFINITY;
+        // log2 units; +inf for rows past the end so that P = 0 there.  A row that saw nothing
+        // but masked keys (bias_log2) stored its row sum n instead: its probabilities are
+        // exp2(x + FLT_MAX) / n.  The kernel works with exp2(x + FLT_MAX) and the true delta,
+        // and applies 1 / n to the finished dQ row and to the delta that it hands on (the dK / dV
+        // kernel scales that row of dO instead).
+        lse2 = row_ok ? (kBias ? lse_reference(lse_raw, kLog2e) : lse_raw * kLog2e) : INFINITY;
+        if constexpr (kBias) inv_n = lse_row_factor(lse_raw);
         // delta = sum_d dO * O: lanes i and i + 32 hold complementary head-dim slots of row i
         float part = 0.f;
 #pragma unroll
@@ -155,7 +160,7 @@ __global__ __launch_bounds__(kThreads, (kStagger && DPAD > 64 ? 1 : 2)) void att
                 part = __builtin_fmaf((float)gf[t][j], (float)of[j], part);
         }
         delta = sum_xor32(part);  // masked dO slots are zero, so clamped rows / columns add nothing
-        if (row_ok && g == 0) a.delta[(int64_t)bh * a.sq + q_row] = delta;
+        if (row_ok && g == 0) a.delta[(int64_t)bh * a.sq + q_row] = delta * inv_n;
     }
     // Where the registers allow it the per-row terms enter through the accumulators: S^T starts
     // from -lse (log2 units) and, without dropout, dP^T from -delta, in all sixteen registers of
@@ -501,8 +506,8 @@ __global__ __launch_bounds__(kThreads, (kStagger && DPAD > 64 ? 1 : 2)) void att
     if (wq0 < a.sq) {
         T* dq_row0 =
             reinterpret_cast<T*>(a.dq) + b * a.dqs[0] + (int64_t)wq0 * a.dqs[1] + h * a.dqs[2];
-        store_block_via_lds<T, DPAD, kPitch>(dq_acc, a.scale, k_lds + wave * 32 * kPitch, dq_row0,
-                                             a.dqs[1], a.sq - wq0, a.d);
+        store_block_via_lds<T, DPAD, kPitch>(dq_acc, a.scale * inv_n, k_lds + wave * 32 * kPitch,
+                                             dq_row0, a.dqs[1], a.sq - wq0, a.d);
     }
 }
 

@@ -155,11 +155,14 @@ __global__ __launch_bounds__(kBwdThreads, (bwd_two_per_cu(DPAD, kDrop, KB) ? 2 :
         QStage q, g;
         float stat;
         uint32_t mask;
+        float row_lse;  // kBias: lse of tile row (thread & 63), in every wavefront
     };
     TileRegs regs;
     regs.q.init(a.qs[1], a.d);
     regs.g.init(a.os[1], a.d);
     regs.stat = 0.f, regs.mask = 0u;
+    regs.row_lse = 0.f;
+    int masked_pending = 0, masked_tile[2] = {0, 0};  // staged tiles that sync_staged must fix
     // lse / delta of a query tile: threads 0..63 fetch lse, threads 64..127 delta.
     const float* stat_src = (threadIdx.x < kBwdBM) ? lse_base : delta_base;
     // Requests tile t.  Unconditional: rows are clamped into the tensor (past the last tile the
@@ -177,6 +180,7 @@ __global__ __launch_bounds__(kBwdThreads, (bwd_two_per_cu(DPAD, kDrop, KB) ? 2 :
         // 697 us at S 4096) and keeps it.
         if (!(DPAD > 96 && kDrop == 0) || threadIdx.x < 2 * kBwdBM)
             r.stat = stat_src[min(i0 + (int)(threadIdx.x & (kBwdBM - 1)), a.sq - 1)];
+        if constexpr (kBias) r.row_lse = lse_base[min(i0 + (int)(threadIdx.x & 63), a.sq - 1)];
         if constexpr (kDrop == 3) {
             // the keep bits that the forward stored: thread (w, row) of the workgroup fetches the
             // word of query row i0 + row for the 32 keys of wavefront w
@@ -191,6 +195,13 @@ __global__ __launch_bounds__(kBwdThreads, (bwd_two_per_cu(DPAD, kDrop, KB) ? 2 :
         const int i0 = t * kBwdBM;
         r.q.fix(i0, a.sq, a.d);
         r.g.fix(i0, a.sq, a.d);
+        if constexpr (kBias) {
+            // Every wavefront holds the 64 lse values of the tile, one per lane, so all of them
+            // agree on whether the tile has a row that saw nothing but masked keys; see
+            // sync_staged for what happens then.
+            if (__builtin_amdgcn_ballot_w64(masked_row_lse(r.row_lse)) != 0)
+                masked_pending |= 1 << buf, masked_tile[buf] = t;
+        }
         r.q.store(q_lds + buf * SM::kQTile);
         r.g.store(g_lds + buf * SM::kQTile);
         if (threadIdx.x < 2 * kBwdBM) {
@@ -199,12 +210,42 @@ __global__ __launch_bounds__(kBwdThreads, (bwd_two_per_cu(DPAD, kDrop, KB) ? 2 :
             // P = 0 there) and, without dropout, -delta; kept at row_slot so that one 128-bit
             // read returns the values of four accumulator registers in order
             const float v = (threadIdx.x < kBwdBM)
-                                ? (ok ? -(r.stat * kLog2e) : -INFINITY)
+                                ? (ok ? -(kBias ? lse_reference(r.stat, kLog2e) : r.stat * kLog2e)
+                                      : -INFINITY)
                                 : (ok ? (kDrop == 0 ? -r.stat : r.stat) : 0.f);
             stat_lds[buf * 2 * kBwdBM + (threadIdx.x & kBwdBM) + row_slot(threadIdx.x & (kBwdBM - 1))] = v;
         }
         if constexpr (kDrop == 3)
             mask_lds[buf * kBwdThreads + (threadIdx.x & ~63) + row_slot(threadIdx.x & 63)] = r.mask;
+    };
+    // The barrier after a stage_tile.  Rows that saw nothing but masked keys (bias_log2) have
+    // probabilities exp2(x + FLT_MAX) / n: the division goes onto their row of dO (and, in the dQ
+    // kernel, onto the delta it stored), which puts it into dV, dP and dS alike.  It is applied to
+    // the staged tile in LDS, each thread on the chunks it wrote, behind a test that is uniform
+    // over the workgroup and false for every tile of an ordinary call.
+    auto sync_staged = [&]() __attribute__((always_inline)) {
+        __syncthreads();
+        if constexpr (kBias) {
+            if (__builtin_expect(masked_pending != 0, 0)) {
+#pragma unroll 1
+                for (int buf = 0; buf < 2; ++buf) {
+                    if (!(masked_pending >> buf & 1)) continue;
+                    const int i0 = masked_tile[buf] * kBwdBM;
+                    T* tile = g_lds + buf * SM::kQTile;
+#pragma unroll
+                    for (int u = 0; u < QStage::kPerThread; ++u) {
+                        const int c = threadIdx.x + u * kBwdThreads;
+                        if (QStage::kChunks % kBwdThreads != 0 && c >= QStage::kChunks) continue;
+                        const int row = c / QStage::kChunksPerRow, cc = c % QStage::kChunksPerRow;
+                        const float f = lse_row_factor(lse_base[min(i0 + row, a.sq - 1)]);
+                        u32x4_t* p = reinterpret_cast<u32x4_t*>(tile + row * kPitch + cc * 8);
+                        *p = __builtin_bit_cast(u32x4_t, scale_frag<T>(*p, f));
+                    }
+                }
+                masked_pending = 0;
+                __syncthreads();
+            }
+        }
     };
     auto tile_fast = [&](int t) __attribute__((always_inline)) {
         const int i0 = t * kBwdBM;
@@ -237,7 +278,7 @@ __global__ __launch_bounds__(kBwdThreads, (bwd_two_per_cu(DPAD, kDrop, KB) ? 2 :
     if constexpr (kPairGeneric) {
         if (pair_first) stage_tile(second, t_lo + 1);
     }
-    __syncthreads();
+    sync_staged();
 
     // wavefront-uniform: does the 32-query half tile at ih0 see any key of this wavefront?
     auto half_active = [&](int ih0) __attribute__((always_inline)) {
@@ -506,7 +547,7 @@ __global__ __launch_bounds__(kBwdThreads, (bwd_two_per_cu(DPAD, kDrop, KB) ? 2 :
                        std::integral_constant<bool, kLateRequest>{});
         // stage the next query tile (its buffer was last read before the previous barrier)
         if (t + 1 < t_hi) stage_tile(regs, t + 1);
-        __syncthreads();
+        sync_staged();
     };
 
     // Diagonal / window / tail tiles: activity and masks are tested per wavefront and half tile.
@@ -546,19 +587,19 @@ __global__ __launch_bounds__(kBwdThreads, (bwd_two_per_cu(DPAD, kDrop, KB) ? 2 :
             request_tile(regs, t + 1);
             generic_tiles(t, 1);
             if (t + 1 < t_hi) stage_tile(regs, t + 1);
-            __syncthreads();
+            sync_staged();
             return 1;
         }
         if (!(pair_first && t == t_lo)) {  // otherwise the start-up has staged tile t+1 already
             request_tile(regs, t + 1);
             stage_tile(regs, t + 1);  // the other buffer: last read before the previous barrier
-            __syncthreads();
+            sync_staged();
         }
         request_tile(regs, t + 2);
         generic_tiles(t, 2);
         __syncthreads();  // tile t+2 goes where tile t was
         if (t + 2 < t_hi) stage_tile(regs, t + 2);
-        __syncthreads();
+        sync_staged();
         return 2;
     };
     {

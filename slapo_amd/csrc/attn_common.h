@@ -132,13 +132,37 @@ __device__ __forceinline__ float sum2<bf16_t>(uint32_t pair, float acc) {
     return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pair), ones, acc, false);
 }
 
-// An additive bias in log2 units.  Mask values near the most negative finite number (HF-style
-// padding masks use finfo.min) would overflow to -inf under the multiplication; they stay
-// finite, so that a row that sees only such keys keeps a finite, uniform softmax as in the
-// reference.  A true -inf is left alone.
+// Masking values.  A bias at or below kMaskBias (-5e8: "-1e9", also after rounding to bf16,
+// "-1e30", finfo.min of bf16 / fp32 are what models add to hide a key) is taken as THE masking
+// value and becomes -FLT_MAX exactly;
+// a true -inf is left alone.  Added to a score in fp32 such a bias swallows the score in the
+// reference too, so a query row that sees nothing but masked keys gets a uniform softmax over them
+// there and here.  For such a row the kernels keep m = -FLT_MAX as the softmax reference point
+// (masked scores minus it are exactly 0) and the row sum n = number of those keys; the usual
+// log-sum-exp m + log n cannot hold n beside m, so the forward stores n * 2^100 in its place
+// (no real log-sum-exp comes near 6e29) and the backward decodes it: probabilities are
+// exp(x - m) / n.
+constexpr float kMaskBias = -5e8f;
+constexpr float kFltMax = 3.4028234663852886e38f;
+constexpr float kMaskedRowLse = 1.2676506002282294e30f;  // 2^100
+__device__ __forceinline__ float canonical_bias(float b) {
+    return (b <= kMaskBias && b != -INFINITY) ? -kFltMax : b;
+}
+// An additive bias in log2 units.
 __device__ __forceinline__ float bias_log2(float b) {
-    const float v = b * kLog2e;
-    return (v == -INFINITY && b != -INFINITY) ? -3.4028234663852886e38f : v;
+    return (b <= kMaskBias && b != -INFINITY) ? -kFltMax : b * kLog2e;
+}
+// What the forward stores as log-sum-exp of a row with reference point m (any units) and row sum l.
+__device__ __forceinline__ bool masked_row_lse(float lse) {
+    return lse >= 0.5f * kMaskedRowLse && lse < INFINITY;
+}
+// The reference point that exp subtracts for a stored log-sum-exp, times `unit` (1 for natural
+// units, log2(e) for log2 units), and the factor 1 / n that goes with it (1 for ordinary rows).
+__device__ __forceinline__ float lse_reference(float lse, float unit) {
+    return masked_row_lse(lse) ? -kFltMax : lse * unit;
+}
+__device__ __forceinline__ float lse_row_factor(float lse) {
+    return masked_row_lse(lse) ? kMaskedRowLse / lse : 1.0f;
 }
 
 // Fragment of 8 elements times a scalar, rounded back to T.
@@ -389,6 +413,16 @@ struct TileStage {
             const int cc = c % kChunksPerRow;
             if (row0 + row >= n_rows || cc * 8 >= d) r[u] = u32x4_t{0u, 0u, 0u, 0u};
         }
+    }
+    // Chunk u times f[u] (one factor per row that the thread holds a chunk of), rounded back to T.
+    __device__ __forceinline__ void scale_rows(const float (&f)[kPerThread]) {
+#pragma unroll
+        for (int u = 0; u < kPerThread; ++u)
+            r[u] = __builtin_bit_cast(u32x4_t, scale_frag<T>(r[u], f[u]));
+    }
+    // Tile row of chunk u of this thread.
+    static __device__ __forceinline__ int row_of(int u) {
+        return (threadIdx.x + u * THREADS) / kChunksPerRow;
     }
     __device__ __forceinline__ void store(T* lds) const {
 #pragma unroll

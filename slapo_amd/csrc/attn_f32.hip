@@ -16,7 +16,8 @@ constexpr int kRows = 64;   // threads (= owned rows) per block
 constexpr int kTile = 16;   // streamed rows per LDS tile
 
 __device__ __forceinline__ float bias_at(const AttnArgs& a, int b, int h, int i, int j) {
-    return a.bias[b * a.bs[0] + h * a.bs[1] + (int64_t)i * a.bs[2] + (int64_t)j * a.bs[3]];
+    return canonical_bias(
+        a.bias[b * a.bs[0] + h * a.bs[1] + (int64_t)i * a.bs[2] + (int64_t)j * a.bs[3]]);
 }
 
 __device__ __forceinline__ float drop_scale(const AttnArgs& a, int bh, int i, int j) {
@@ -94,7 +95,8 @@ __global__ __launch_bounds__(kRows) void attn_f32_fwd_kernel(const AttnArgs a) {
 #pragma unroll
     for (int c = 0; c < DMAX; ++c)
         if (c < a.d) op[c] = o[c] * inv_l;
-    a.lse[(int64_t)bh * a.sq + i] = m + logf(l);
+    // a row that saw nothing but masked keys: see canonical_bias
+    a.lse[(int64_t)bh * a.sq + i] = m == -kFltMax ? l * kMaskedRowLse : m + logf(l);
 }
 
 // dQ: thread = query.  dq_i = scale * sum_j ds_ij k_j,  ds = p (dp - delta),  dp = dO_i . v_j
@@ -119,7 +121,8 @@ __global__ __launch_bounds__(kRows) void attn_f32_dq_kernel(const AttnArgs a) {
         go[c] = ok ? gp[(int64_t)i * a.os[1] + c] : 0.f;
         dq[c] = 0.f;
     }
-    const float lse = row_ok ? a.lse[(int64_t)bh * a.sq + i] : 0.f;
+    const float lse_raw = row_ok ? a.lse[(int64_t)bh * a.sq + i] : 0.f;
+    const float lse = lse_reference(lse_raw, 1.0f), inv_n = lse_row_factor(lse_raw);
     const float delta = row_ok ? a.delta[(int64_t)bh * a.sq + i] : 0.f;
 
     int j_lo, j_hi;
@@ -141,7 +144,7 @@ __global__ __launch_bounds__(kRows) void attn_f32_dq_kernel(const AttnArgs a) {
                 dp = __builtin_fmaf(go[c], vs[jj][c], dp);
             }
             if (a.has_bias) s += bias_at(a, b, h, i, j);
-            const float p = expf(s - lse);
+            const float p = expf(s - lse) * inv_n;
             if (a.dropout) dp *= drop_scale(a, bh, i, j);
             const float ds = p * (dp - delta);
 #pragma unroll
@@ -162,7 +165,7 @@ template <int DMAX, int kWhich>
 __global__ __launch_bounds__(kRows) void attn_f32_dkv_kernel(const AttnArgs a) {
     __shared__ float qs[kTile][DMAX];
     __shared__ float gs[kTile][DMAX];
-    __shared__ float lse_s[kTile];
+    __shared__ float lse_s[kTile], inv_n_s[kTile];
     __shared__ float delta_s[kTile];
     const int bh = blockIdx.y, b = bh / a.heads, h = bh % a.heads;
     const int k0 = blockIdx.x * kRows;
@@ -190,7 +193,9 @@ __global__ __launch_bounds__(kRows) void attn_f32_dkv_kernel(const AttnArgs a) {
         load_rows<DMAX>(gs, gp, a.os[1], i0, a.sq, a.d);
         if (threadIdx.x < kTile) {
             const int i = i0 + threadIdx.x;
-            lse_s[threadIdx.x] = i < a.sq ? a.lse[(int64_t)bh * a.sq + i] : 0.f;
+            const float lse_raw = i < a.sq ? a.lse[(int64_t)bh * a.sq + i] : 0.f;
+            lse_s[threadIdx.x] = lse_reference(lse_raw, 1.0f);
+            inv_n_s[threadIdx.x] = lse_row_factor(lse_raw);
             delta_s[threadIdx.x] = i < a.sq ? a.delta[(int64_t)bh * a.sq + i] : 0.f;
         }
         __syncthreads();
@@ -203,7 +208,7 @@ __global__ __launch_bounds__(kRows) void attn_f32_dkv_kernel(const AttnArgs a) {
 #pragma unroll
             for (int c = 0; c < DMAX; ++c) s = __builtin_fmaf(qs[ii][c], kr[c], s);
             if (a.has_bias) s += bias_at(a, b, h, i, j);
-            const float p = expf(s - lse_s[ii]);
+            const float p = expf(s - lse_s[ii]) * inv_n_s[ii];
             const float keep = a.dropout ? drop_scale(a, bh, i, j) : 1.f;
             if (kWhich == 1) {
                 const float pd = p * keep;

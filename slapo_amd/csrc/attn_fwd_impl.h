@@ -118,7 +118,6 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
         for (int r = 0; r < 16; ++r) o_acc[x][r] = 0.f;
     // Softmax state of this lane's query, in log2 units (Q carries scale * log2(e)): m_run is the
     // reference point of l_run / o_acc (-inf: nothing accumulated yet), moved lazily.
-    constexpr float kHugeNeg = -1e30f;
     float m_run = -INFINITY;
     float m_ref = 0.f;  // what the exponentials subtract: m_run, or 0 while m_run is -inf
     float l_run = 0.f;  // this lane's share of the running sum
@@ -234,8 +233,8 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
     };
     // Moves the reference point if this tile's maximum calls for it (rare after a row's first
     // tile): only when the maximum exceeds it by more than kMaxSlack, so that the rescale of the
-    // accumulators stays off the common path.  A row that has met nothing but keys masked with a
-    // huge negative bias sits at that value and moves up to the first real key like any other.
+    // accumulators stays off the common path.  A row that has met nothing but masked keys
+    // sits at -FLT_MAX and moves up to the first real key like any other.
     auto update_reference = [&](float mx) __attribute__((always_inline)) {
         const bool move = mx > m_run + kMaxSlack && mx != -INFINITY;
         if (__builtin_expect(__builtin_amdgcn_ballot_w64(move) != 0, 0)) {
@@ -448,13 +447,12 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
                                              a.os[1], a.sq - wq0, a.d);
     }
     if (q_row < a.sq) {
-        // A row that met nothing but keys masked with a huge negative bias has a uniform softmax
-        // here (as in the reference) but no log-sum-exp that fp32 can hold next to its scores:
-        // +inf is stored, which makes the backward treat the row as contributing no gradient.
+        // A row that met nothing but masked keys (bias_log2) sits at -FLT_MAX with l_tot = their
+        // number: the row sum goes out in place of the log-sum-exp, scaled by 2^100.
         if (g == 0)
-            a.lse[(int64_t)bh * a.sq + q_row] = (m_run > kHugeNeg || m_run == -INFINITY)
-                                                    ? (m_run + __builtin_log2f(l_tot)) * kLn2
-                                                    : INFINITY;
+            a.lse[(int64_t)bh * a.sq + q_row] = m_run == -kFltMax
+                                                    ? l_tot * kMaskedRowLse
+                                                    : (m_run + __builtin_log2f(l_tot)) * kLn2;
     }
 }
 

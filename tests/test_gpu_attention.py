@@ -151,36 +151,46 @@ def test_padding_masks_and_tile_skipping(dtype, causal, kind):
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
 @pytest.mark.parametrize("d", [64, 80, 128])
-def test_rows_that_see_only_masked_keys(dtype, d):
+@pytest.mark.parametrize("neg,layout,p", [
+    (None, "b11k", 0.0),    # finfo(dtype).min, the HF padding mask as it arrives
+    (-1e9, "b11k", 0.0),    # the other constant that models use
+    (None, "bhqk", 0.0),    # the same mask expanded over heads and queries (bias read per score)
+    (-1e30, "b11k", 0.2),   # with dropout
+])
+def test_rows_that_see_only_masked_keys(dtype, d, neg, layout, p):
     """Left padding under a causal mask (the batch layout of generation with HF models): the first
-    rows of a sequence see nothing but keys masked with finfo.min.  The reference adds the mask
-    in floating point, the masked scores swallow the raw ones and the softmax of such a row is
-    finite and uniform; so it is here (no NaN may reach the rows after them).  Rows that see a
-    real key must match the oracle in every output; the masked-only rows are compared in the
-    forward, and their gradient contribution is finite (zero by construction on the MFMA path
-    for masks of the bf16 / fp32 magnitude, the oracle's value otherwise)."""
+    rows of a sequence see nothing but masked keys.  The reference adds the mask in floating
+    point, the masked scores swallow the raw ones and the softmax of such a row is finite and
+    uniform over the keys it may see; so it is here, in the forward and in every gradient (no
+    NaN may reach the rows after them, and the upstream gradient of the padded rows flows like
+    the oracle's)."""
     b, s, h = 3, 320, 2
     q, k, v, do, g = _inputs(b, s, h, d, dtype)
-    neg = torch.finfo(dtype).min
+    neg = torch.finfo(dtype).min if neg is None else neg
     m = torch.zeros(b, 1, 1, s)
     pads = (5, 64, 200)
     for i, n in enumerate(pads):
         m[i, 0, 0, :n] = neg
-    mask = m.to(dtype)
-    out, dq, dk, dv = _run(q, k, v, do, mask, True)
-    assert torch.isfinite(out).all() and torch.isfinite(dq).all()
-    assert torch.isfinite(dk).all() and torch.isfinite(dv).all()
-    ro = OA.xformers_ref(q, k, v, mask, True, compute_dtype=torch.float64)
-    assert_parity(out, ro, dtype, "out")
-    # gradients: feed only the rows that see a real key, so that both sides agree on what flows
-    do2 = do.clone()
-    for i, n in enumerate(pads):
-        do2[i, :n] = 0
-    out, dq, dk, dv = _run(q, k, v, do2, mask, True)
-    _, rq, rk, rv = OA.attention_fwd_bwd(q, k, v, do2, mask, True, 0, 0.0, None, None,
-                                         torch.float64)
-    for name, a, r in (("dq", dq, rq), ("dk", dk, rk), ("dv", dv, rv)):
+    mask = m.to(torch.float32 if abs(neg) > 1e5 and dtype == torch.float16 else dtype)
+    if layout == "bhqk":
+        mask = mask.expand(b, h, s, s).contiguous()
+    out, dq, dk, dv = _run(q, k, v, do, mask, True, 0, p)
+    for t in (out, dq, dk, dv):
+        assert torch.isfinite(t).all()
+    keep = _torch_keep(b, h, s, s, p) if p > 0 else None
+    # -1e9 swallows the scores in the reference's fp32 / bf16 arithmetic but not in fp64
+    compute = torch.float32 if neg == -1e9 else torch.float64
+    ro, rq, rk, rv = OA.attention_fwd_bwd(q, k, v, do, mask.float(), True, 0, p, keep, None,
+                                          compute)
+    for name, a, r in (("out", out, ro), ("dq", dq, rq), ("dk", dk, rk), ("dv", dv, rv)):
         assert_parity(a, r, dtype, name)
+    if dtype == torch.float16 and abs(neg) < 1e5:
+        return  # -65504 does not swallow the scores: nothing below applies
+    # the padded rows themselves: uniform attention over the keys they may see
+    vd = torch.ones_like(v)
+    out1 = _run(q, k, vd, do, mask, True)[0]
+    for i, n in enumerate(pads):
+        assert (out1[i, :n].float() - 1.0).abs().max() <= 2e-2
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
