@@ -123,6 +123,8 @@ int fill_args(const slapo_attn_params* p, AttnArgs* a, bool backward) {
     if ((int64_t)p->batch * p->heads > 0x7FFFFFFF / 2) return SLAPO_ERR_SHAPE;
     if (!(p->p_drop >= 0.f && p->p_drop <= 1.f)) return SLAPO_ERR_ARG;
     if (p->window < 0) return SLAPO_ERR_ARG;
+    // the scale is folded into Q / K fragments: a NaN or infinite one would poison every score
+    if (!(p->scale > -kFltMax && p->scale < kFltMax)) return SLAPO_ERR_ARG;
     const bool half = p->dtype == SLAPO_F16 || p->dtype == SLAPO_BF16;
     if (!half && p->dtype != SLAPO_F32) return SLAPO_ERR_DTYPE;
     if (half) {

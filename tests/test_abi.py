@@ -141,6 +141,10 @@ def test_compute_entry_points_validate_before_touching_the_device():
     prm.p_drop = 0.5  # dropout without a valid plan
     assert lib.slapo_amd_attn_fwd(ctypes.byref(prm), 16, 16, 16, None, 16, 16, None) == -4
     prm.p_drop, prm.dtype = 0.0, 1
+    for bad in (float("nan"), float("inf"), -float("inf")):  # a softmax scale that is no number
+        prm.scale = bad
+        assert lib.slapo_amd_attn_fwd(ctypes.byref(prm), 16, 16, 16, None, 16, 16, None) == -4
+    prm.scale = 0.125
     assert lib.slapo_amd_attn_bwd_workspace_bytes(ctypes.byref(prm)) == 8 * 4
     # keep-bit buffer: one uint32 per (batch*head, 32 keys, query rounded up to 4); none without
     # dropout or for fp32
