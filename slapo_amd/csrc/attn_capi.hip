@@ -99,9 +99,13 @@ __global__ __launch_bounds__(256) void keep_mask_kernel(const AttnArgs a) {
     a.keep_mask[((int64_t)bh * a.mask_words + w) * a.mask_pitch + i] = word;
 }
 
+// (grid limits of keep_mask_kernel: one grid row per word of 32 keys, one grid plane per head)
+bool keep_mask_kernel_fits(const AttnArgs& a) {
+    return a.mask_words <= 65535 && (int64_t)a.batch * a.heads <= 65535;
+}
 int draw_keep_mask(const AttnArgs& a, hipStream_t st) {
     const int64_t bh = (int64_t)a.batch * a.heads;
-    if (a.mask_words > 65535 || bh > 65535) return SLAPO_ERR_SHAPE;
+    if (!keep_mask_kernel_fits(a)) return SLAPO_ERR_SHAPE;
     const dim3 grid((unsigned)((a.sq + 255) / 256), (unsigned)a.mask_words, (unsigned)bh);
     if (a.dropout == 1)
         hipLaunchKernelGGL(keep_mask_kernel<false>, grid, dim3(256), 0, st, a);
@@ -209,7 +213,7 @@ extern "C" int slapo_amd_attn_fwd(const slapo_attn_params* prm, const void* q, c
     hipStream_t st = (hipStream_t)stream;
     if (prm->dtype == SLAPO_F32) return attn_fwd_f32(a, st);
     if (!half_ptrs_ok({q, k, v, o})) return SLAPO_ERR_ALIGN;
-    if (a.dropout && a.keep_mask && a.window > 0) {
+    if (a.dropout && a.keep_mask && a.window > 0 && keep_mask_kernel_fits(a)) {
         // Local window with a buffer for the keep bits: draw them first, the forward kernel
         // then reads them like the backward kernels do (bf16 B4 S2048 H16 D128, window 256,
         // p 0.1: 88 against 127 us).  Without a window the forward draws them itself and
