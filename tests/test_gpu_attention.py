@@ -366,6 +366,20 @@ def test_attention_dropout_over_several_philox_trips(dtype):
     _check(q, k, v, do, None, True, 0, dtype, p=p)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("d,window", [(64, 0), (128, 0), (128, 40)])
+def test_dropout_probability_one(dtype, d, window):
+    """p = 1 drops everything: zero output and zero gradients, as F.dropout(p=1) gives the
+    reference, and the generator is left alone."""
+    q, k, v, do, _ = _inputs(2, 130, 2, d, dtype)
+    torch.cuda.manual_seed(11)
+    before = torch.cuda.get_rng_state()
+    out, dq, dk, dv = _run(q, k, v, do, None, True, window, 1.0, seed=11)
+    assert torch.equal(torch.cuda.get_rng_state(), before)
+    for t in (out, dq, dk, dv):
+        assert torch.count_nonzero(t) == 0
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("d,scale", [(80, 1.0), (128, 1.0), (128, 0.01), (64, 0.0), (80, -0.05)])
 def test_softmax_scale_other_than_the_default(dtype, d, scale):
