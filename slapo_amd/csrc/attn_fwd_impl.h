@@ -476,8 +476,11 @@ template <typename T, int DPAD, int kWin>
 int dispatch_nobias(const AttnArgs& a, hipStream_t st) {
     if (a.dropout == 1) return launch<T, DPAD, 0, 1, kWin>(a, st);
     if (a.dropout == 2) return launch<T, DPAD, 0, 2, kWin>(a, st);
-    if constexpr (kWin != 0) {  // stored keep bits: local-window calls only, see attn_capi.hip
-        if (a.dropout == 3) return launch<T, DPAD, 0, 3, kWin>(a, st);
+    if (a.dropout == 3) {  // stored keep bits: local-window calls only, see attn_capi.hip
+        if constexpr (kWin != 0)
+            return launch<T, DPAD, 0, 3, kWin>(a, st);
+        else
+            return SLAPO_ERR_ARG;
     }
     return launch<T, DPAD, 0, 0, kWin>(a, st);
 }
