@@ -164,6 +164,16 @@ class FlashAttentionOp(nn.Module):
                 f"scale={self.scale}, window={self.window}")
 
 
+def _has_hooks(module):
+    """True if any per-module or global forward / backward hook would run on `module(...)`."""
+    # pylint: disable=protected-access
+    from torch.nn.modules import module as M
+    return bool(module._forward_hooks or module._forward_pre_hooks or module._backward_hooks
+                or module._backward_pre_hooks or M._global_forward_hooks
+                or M._global_forward_pre_hooks or M._global_backward_hooks
+                or M._global_backward_pre_hooks)
+
+
 class FlashAttention(nn.Module):
     """HF-style self-attention block: QKV projection(s) -> FlashAttentionOp -> optional output
     projection + residual dropout.  Restrictions are the reference's: no cross attention, no
@@ -223,6 +233,18 @@ class FlashAttention(nn.Module):
         return tuple(self.reshape_for_scores(proj(hidden_states))
                      for proj in (self.query, self.key, self.value))
 
+    def _tail_can_fuse(self, x):
+        """The fused out_proj-bias + resid_dropout pass stands in for the two child calls only when
+        nothing could tell the difference: both children are the plain torch modules, carry no
+        hooks (a schedule's `.sync(mode="fwd_post")` is a forward hook on `out_proj`,
+        slapo/sharding/shard_ops.py:436-440; `.replace` moves hooks along, primitives/replace.py:254),
+        and the input is a real device tensor (not an fx Proxy during tracing)."""
+        proj, drop = self.out_proj, self.resid_dropout
+        return (type(x) is torch.Tensor and x.is_cuda
+                and type(proj) is nn.Linear and proj.bias is not None
+                and type(drop) is nn.Dropout and not drop.inplace
+                and not _has_hooks(proj) and not _has_hooks(drop))
+
     def forward(
         self,
         hidden_states: Optional[tuple[torch.FloatTensor]],
@@ -257,11 +279,10 @@ class FlashAttention(nn.Module):
         context_layer = context_layer.view(context_layer.size()[:-2] + (-1,))
 
         if self.output_proj:
-            # out_proj's bias and resid_dropout ride on one pass over [B, S, hidden] (the reference
-            # runs the GEMM with bias, then nn.Dropout: slapo/op/attention.py:514-516).  The mask
-            # is the one nn.Dropout would draw; p and training are read from the child module, so
-            # schedules that edit `resid_dropout` keep working.
-            if self.out_proj.bias is not None:
+            if self._tail_can_fuse(context_layer):
+                # out_proj's bias and resid_dropout ride on one pass over [B, S, hidden] (the
+                # reference runs the GEMM with bias, then nn.Dropout: slapo/op/attention.py:514-516).
+                # The mask is the one nn.Dropout would draw; p and training are read from the child.
                 context_layer = bias_dropout(
                     F.linear(context_layer, self.out_proj.weight, None), self.out_proj.bias,
                     self.resid_dropout.p, self.resid_dropout.training)

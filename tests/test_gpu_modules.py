@@ -71,3 +71,83 @@ def test_window_kwarg_local_attention_module():
     out_g, _ = mg(x)
     # the first `window` positions see the same keys under both masks, later ones do not
     assert torch.equal(out[:, :16], out_g[:, :16]) and not torch.equal(out[:, 16:], out_g[:, 16:])
+
+
+def _attention_with_dropout_tail():
+    torch.manual_seed(3)
+    m = op.FlashAttention(hidden_size=256, num_attention_heads=4, output_proj=True,
+                          attn_pdrop=0.0, resid_pdrop=0.1, attn_op_name="hip_cdna4",
+                          fused_qkv=True).half().cuda()
+    x = torch.randn(2, 128, 256, dtype=torch.float16, device="cuda")
+    return m, x
+
+
+def _same_mask_close_values(a, b):
+    assert ((a == 0) != (b == 0)).float().mean().item() < 5e-4  # exact zeros of the GEMM aside
+    assert 0.08 < (a == 0).float().mean().item() < 0.12
+    torch.testing.assert_close(a.float(), b.float(), atol=1e-2, rtol=1e-2)
+
+
+def test_hooks_on_out_proj_fire_and_their_result_is_used():
+    """Schedules hang the tensor-parallel all-reduce on `out_proj` as a forward hook
+    (`.sync(mode="fwd_post")`: slapo/sharding/shard_ops.py:436-440, model_schedule/gpt2.py:482-485)
+    and `.replace` carries hooks over (primitives/replace.py:254).  With a hook on either child the
+    block calls the children as the reference does (attention.py:514-516): the hook runs once per
+    forward and what it returns is what `resid_dropout` sees.  Without hooks the fused pass runs
+    and draws the same mask as `nn.Dropout`."""
+    m, x = _attention_with_dropout_tail()
+    torch.cuda.manual_seed(77)
+    plain, _ = m(x)
+
+    calls = []
+
+    def post(mod, inp, out):
+        calls.append(tuple(out.shape))
+        return out * 2
+
+    h = m.out_proj.register_forward_hook(post)
+    torch.cuda.manual_seed(77)
+    hooked, _ = m(x)
+    assert calls == [(2, 128, 256)]
+    # the same draw masks both paths; values differ by the roundings of GEMM-with-bias then
+    # dropout against GEMM then bias + dropout in one pass
+    _same_mask_close_values(hooked, plain * 2)
+    h.remove()
+
+    pre_calls = []
+    h = m.out_proj.register_forward_pre_hook(lambda mod, inp: pre_calls.append(1))
+    torch.cuda.manual_seed(77)
+    again, _ = m(x)
+    assert pre_calls == [1]
+    _same_mask_close_values(again, plain)
+    h.remove()
+
+    grads = []
+    h = m.out_proj.register_full_backward_hook(lambda mod, gi, go: grads.append(go[0].shape))
+    xg = x.clone().requires_grad_(True)
+    m(xg)[0].sum().backward()
+    assert len(grads) == 1
+    h.remove()
+
+
+def test_replaced_children_of_the_tail_are_called_as_modules():
+    """A `resid_dropout` replaced by Identity (no `.p`) or an `out_proj` wrapped in another module
+    type must keep working: the block then calls them as the reference does."""
+    m, x = _attention_with_dropout_tail()
+    torch.cuda.manual_seed(5)
+    fused, _ = m(x)
+    m.resid_dropout = torch.nn.Identity()
+    no_drop, _ = m(x)
+    kept = fused != 0
+    assert torch.allclose(fused[kept].float(), no_drop[kept].float() / 0.9, atol=2e-3, rtol=2e-3)
+
+    class Wrapped(torch.nn.Module):
+        def __init__(self, inner):
+            super().__init__()
+            self.inner = inner
+
+        def forward(self, t):
+            return self.inner(t) + 1
+
+    m.out_proj = Wrapped(m.out_proj)
+    assert torch.equal(m(x)[0], no_drop + 1)

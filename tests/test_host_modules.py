@@ -287,3 +287,43 @@ def test_checkpoint_replays_every_random_stream(monkeypatch):
     out = ckpt.checkpoint(lambda t: (t @ w1).relu(), x, use_reentrant=False)
     out.sum().backward()
     assert x.grad is not None and w1.grad is not None
+
+
+def test_flash_attention_is_fx_traceable_with_the_op_as_a_leaf():
+    """The GPT-2 schedule traces the replaced attention module with FlashAttentionOp as a leaf and
+    these concrete_args (model_schedule/gpt2.py:457-469); the graph must call the `out_proj` and
+    `resid_dropout` children as modules, so that `.sync` hooks and `.shard` still find them."""
+    from torch import fx
+
+    class _Tracer(fx.Tracer):
+        def is_leaf_module(self, m, qualname):
+            return "FlashAttentionOp" in type(m).__name__ or super().is_leaf_module(m, qualname)
+
+    m = op.FlashAttention(hidden_size=64, num_attention_heads=4, output_proj=True, attn_pdrop=0.1,
+                          resid_pdrop=0.1, attn_op_name="hip_cdna4", fused_qkv=True)
+    graph = _Tracer().trace(m, concrete_args={
+        "layer_past": None, "head_mask": None, "encoder_hidden_states": None,
+        "encoder_attention_mask": None, "use_cache": False, "output_attentions": False})
+    targets = [n.target for n in graph.nodes if n.op == "call_module"]
+    assert targets == ["qkv", "attn_op", "out_proj", "resid_dropout"]
+
+
+def test_fused_tail_is_taken_only_for_plain_hook_free_children():
+    """`_tail_can_fuse` decides between one fused pass and the two child calls of the reference
+    (slapo/op/attention.py:514-516).  Evaluated on the host with a stand-in for a device tensor's
+    `is_cuda`: the decision reads only types and hook tables."""
+    m = op.FlashAttention(64, 4, resid_pdrop=0.1, fused_qkv=True)
+    x = torch.zeros(1, 2, 64)
+    assert m._tail_can_fuse(x) is False  # CPU tensor: the children raise the device error
+    from slapo_amd.op.attention import _has_hooks
+    assert not _has_hooks(m.out_proj) and not _has_hooks(m.resid_dropout)
+    h = m.out_proj.register_forward_hook(lambda mod, inp, out: out)
+    assert _has_hooks(m.out_proj)
+    h.remove()
+    assert not _has_hooks(m.out_proj)
+    h = m.resid_dropout.register_forward_pre_hook(lambda mod, inp: None)
+    assert _has_hooks(m.resid_dropout)
+    h.remove()
+    h = m.out_proj.register_full_backward_hook(lambda mod, gi, go: None)
+    assert _has_hooks(m.out_proj)
+    h.remove()
