@@ -76,8 +76,9 @@ __global__ __launch_bounds__(kBwdThreads, (bwd_two_per_cu(DPAD, kDrop, KB) ? 2 :
     uint32_t* mask_lds = reinterpret_cast<uint32_t*>(smem_raw + 2 * SM::kQBytes + SM::kStatBytes);
 
     const int n_bh = a.batch * a.heads;
-    const int bh = blockIdx.x % n_bh;
-    const int kt = blockIdx.x / n_bh;  // low key tiles see the most queries under a causal mask
+    const int work = work_index(a);
+    const int bh = work % n_bh;
+    const int kt = work / n_bh;  // low key tiles see the most queries under a causal mask
     const int b = bh / a.heads;
     const int h = bh % a.heads;
     const int k0 = kt * kBN;
@@ -639,7 +640,9 @@ int launch(const AttnArgs& a, hipStream_t st) {
     static std::atomic<uint64_t> lds_ready{0};  // per instantiation, one bit per device
     if (allow_dynamic_lds(reinterpret_cast<const void*>(kern), smem, lds_ready) != SLAPO_OK)
         return SLAPO_ERR_LAUNCH;
-    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kBwdThreads), smem, st, a);
+    AttnArgs ordered = a;
+    set_dispatch_order(&ordered, blocks, bwd_two_per_cu(DPAD, kDrop, KB) ? 2 : 1);
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kBwdThreads), smem, st, ordered);
     return check_launch();
 }
 

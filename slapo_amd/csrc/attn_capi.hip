@@ -114,6 +114,20 @@ int draw_keep_mask(const AttnArgs& a, hipStream_t st) {
     return check_launch();
 }
 
+// Compute units of the current device (0 if the runtime will not say), asked once per device.
+int cus_of_current_device() {
+    static std::atomic<int> known[64];
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+    int n = known[dev].load(std::memory_order_relaxed);
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess)
+            return 0;
+        known[dev].store(n, std::memory_order_relaxed);
+    }
+    return n;
+}
+
 bool strides_ok(const int64_t s[3], int mult) {
     return s[0] % mult == 0 && s[1] % mult == 0 && s[2] % mult == 0;
 }
@@ -165,6 +179,8 @@ int fill_args(const slapo_attn_params* p, AttnArgs* a, bool backward) {
     } else {
         a->rng = DropoutState{};
     }
+    a->snake_len = 0, a->snake_rows = 0;
+    a->n_cus = half ? cus_of_current_device() : 0;
     a->keep_mask = nullptr;
     a->mask_words = (p->seqlen_k + 31) / 32;
     a->mask_pitch = (p->seqlen_q + 3) & ~3;

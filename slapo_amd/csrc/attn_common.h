@@ -245,7 +245,42 @@ struct AttnArgs {
     int mask_words, mask_pitch;
     float scale, scale_log2;
     DropoutState rng;
+    // Dispatch order, see work_index: the first `snake_rows` rows of `snake_len` workgroups each
+    // are walked in alternating directions.  n_cus is host-side only (0: unknown).
+    int snake_len, snake_rows;
+    int n_cus;
 };
+
+// Which unit of work a workgroup takes.  The kernels order their work heaviest first (under a
+// causal mask a workgroup's loop has 2 to 2 S / 128 tiles), and the hardware hands the
+// first workgroups out one per CU, row after row of n_cus workgroups, until every CU holds as
+// many as fit; the rest follow as workgroups finish.  With every row in descending order the CU
+// that got the heaviest workgroup of row 0 also gets the heaviest of rows 1, 2: at fp16 B8
+// S1024 H16 D64 half of the CUs then hold 16 + 12 tiles of the dK/dV kernel and the other half
+// 14 + 10, the latter get the next-heaviest workgroups as well, and the launch ends with CUs at
+// 34 to 40 tiles (43 to 53 us).  Walking the odd rows backwards (in groups of eight, so that a
+// workgroup stays on the XCD it would have had: workgroup i runs on XCD i % 8, and the heads are
+// spread over the XCDs the same way) evens the sums out.
+__device__ __forceinline__ int work_index(const AttnArgs& a) {
+    int idx = (int)blockIdx.x;
+    if (a.snake_rows > 0) {
+        const int row = idx / a.snake_len;
+        if (row < a.snake_rows && (row & 1)) {
+            const int pos = idx - row * a.snake_len;
+            idx = row * a.snake_len + (a.snake_len / 8 - 1 - pos / 8) * 8 + (pos & 7);
+        }
+    }
+    return idx;
+}
+// Host: `per_cu` workgroups of the kernel fit a CU at a time; rows that the grid does not fill
+// are left alone.
+inline void set_dispatch_order(AttnArgs* a, int64_t blocks, int per_cu) {
+    a->snake_len = a->n_cus & ~7;
+    a->snake_rows = 0;
+    if (a->snake_len < 8 || !a->causal) return;
+    const int64_t full_rows = blocks / a->snake_len;
+    a->snake_rows = (int)(full_rows < per_cu ? full_rows : per_cu);
+}
 
 __device__ __forceinline__ bool key_visible(const AttnArgs& a, int i, int j) {
     return j < a.sk && (!a.causal || j <= i) && (a.window <= 0 || i - j < a.window);

@@ -61,8 +61,9 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
 
     const int n_bh = a.batch * a.heads;
     const int n_qt = (a.sq + kBM - 1) / kBM;
-    const int bh = blockIdx.x % n_bh;
-    const int qt = n_qt - 1 - blockIdx.x / n_bh;  // heaviest (latest) query tiles first
+    const int work = work_index(a);
+    const int bh = work % n_bh;
+    const int qt = n_qt - 1 - work / n_bh;  // heaviest (latest) query tiles first
     const int b = bh / a.heads;
     const int h = bh % a.heads;
     const int q0 = qt * kBM;
@@ -468,7 +469,9 @@ int launch(const AttnArgs& a, hipStream_t st) {
     static std::atomic<uint64_t> lds_ready{0};  // per instantiation, one bit per device
     if (allow_dynamic_lds(reinterpret_cast<const void*>(kern), smem, lds_ready) != SLAPO_OK)
         return SLAPO_ERR_LAUNCH;
-    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kThreads), smem, st, a);
+    AttnArgs ordered = a;
+    set_dispatch_order(&ordered, blocks, (DPAD <= 64 && kDrop == 0) ? 3 : 2);
+    hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kThreads), smem, st, ordered);
     return check_launch();
 }
 
