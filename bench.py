@@ -22,9 +22,12 @@ cpu_baseline  the oracle's native-PyTorch restatement (fp32 CPU, autograd backwa
           host cores on a bounded sample of the same workload; every epilogue / other_attention
           entry carries a cpu_baseline of its own (a bounded chunk of its tensors)
 
-The headline is the MEDIAN of `--repeats` (default 5) timed loops of `--steps` steps each, every
-loop bracketed by a device synchronisation on both sides; `ms_per_step` x `steps` is the duration
-of that median loop.
+The headline is the MEDIAN of `--repeats` (default 25) timed loops of `--steps` steps each,
+every loop bracketed by a device synchronisation on both sides and free of events; `ms_per_step` x
+`steps` is the duration of that median loop, `median_loop_index` says which one it was (loops are
+listed in the order they ran: a 20-step loop lasts under 3 ms, and the first ones run on clocks
+that have not settled).  The per-kernel durations come from a separate pass over the same steps
+with HIP events around every launch, less the stream time of one event (read between steps).
 """
 from __future__ import annotations
 
@@ -529,7 +532,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--repeats", type=int, default=5,
+    ap.add_argument("--repeats", type=int, default=25,
                     help="timed loops of --steps steps; the median loop is reported")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-epilogues", action="store_true")
@@ -560,25 +563,33 @@ def main():
     for _ in range(args.warmup):
         step.step()
     torch.cuda.synchronize()
-    # Per-kernel durations come from HIP events around the three launches of every fourth step of
-    # the timed region: an event between two kernels costs about 1 us of stream time, which at
-    # 150 us per step would show in `value` if every step carried four of them.
-    every = 4
-    events = [[torch.cuda.Event(enable_timing=True) for _ in range(4)]
-              for _ in range((args.steps + every - 1) // every)]
     loops = []
     for _ in range(max(1, args.repeats)):
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for i in range(args.steps):
-            step.step(events[i // every] if i % every == 0 else None)
+        for _ in range(args.steps):
+            step.step()
         torch.cuda.synchronize()
         loops.append(time.perf_counter() - t0)
-        torch.cuda.synchronize()
-        seg = [sum(ev[i].elapsed_time(ev[i + 1]) for ev in events) / len(events) for i in range(3)]
-        loops[-1] = (loops[-1], seg)
-    loops.sort(key=lambda t: t[0])
-    elapsed, seg_ms = loops[len(loops) // 2]
+    order = sorted(range(len(loops)), key=lambda i: loops[i])
+    median_index = order[len(order) // 2]
+    elapsed = loops[median_index]
+
+    # Per-kernel durations: a pass of its own over the same steps, with HIP events (recorded on the
+    # launching stream) around each of the three launches of every step.  An event between two
+    # launches costs stream time of its own; that cost is read where no kernel runs -- between the
+    # last event of a step and the first event of the next -- and taken off each interval, so that
+    # the three figures add up to a step without events.
+    n_ev = max(args.steps, 40)
+    events = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(n_ev)]
+    torch.cuda.synchronize()
+    for ev in events:
+        step.step(ev)
+    torch.cuda.synchronize()
+    gaps = sorted(events[i][3].elapsed_time(events[i + 1][0]) for i in range(n_ev - 1))
+    event_gap_ms = gaps[len(gaps) // 2]
+    seg_raw = [sum(ev[i].elapsed_time(ev[i + 1]) for ev in events) / len(events) for i in range(3)]
+    seg_ms = [max(t - event_gap_ms, 0.0) for t in seg_raw]
 
     n_pairs = _pairs(cfg["seq"], cfg["causal"]) * cfg["batch"] * cfg["heads"]
     d = cfg["head_dim"]
@@ -602,7 +613,8 @@ def main():
         "warmup": args.warmup,
         "repeats": len(loops),
         "ms_per_step": ms_per_step,
-        "ms_per_step_of_every_loop": [t / args.steps * 1e3 for t, _ in loops],
+        "median_loop_index": median_index,
+        "ms_per_step_of_every_loop": [t / args.steps * 1e3 for t in loops],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -617,6 +629,9 @@ def main():
                      "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / MFMA_PEAK_TFLOPS, "traffic": DKDV_TRAFFIC_BYTES,
                      "flops_per_launch": bwd_flops, "avg_launch_ms": kern_ms},
+        "kernel_timing": {"steps_with_events": n_ev, "event_cost_ms": event_gap_ms,
+                          "raw_event_intervals_ms": seg_raw,
+                          "sum_of_kernels_ms": sum(seg_ms)},
     }
     result["kernels"] = [kern("attn_fwd_kernel<f16,64,0,0,0>", 4 * d * n_pairs, seg_ms[0]),
                          kern("attn_bwd_kernel<f16,64,0,0,1> (dK/dV)", bwd_flops, seg_ms[2]),

@@ -525,7 +525,7 @@ int launch(const AttnArgs& a, hipStream_t st) {
     if (allow_dynamic_lds(reinterpret_cast<const void*>(kern), smem, lds_ready) != SLAPO_OK)
         return SLAPO_ERR_LAUNCH;
     AttnArgs ordered = a;
-    set_dispatch_order(&ordered, blocks, (kStagger && DPAD > 64) ? 1 : 2);
+    set_dispatch_order(&ordered, blocks, (kStagger && DPAD > 64) ? 1 : 2, true);
     hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kThreads), smem, st, ordered);
     return check_launch();
 }

@@ -248,6 +248,9 @@ struct AttnArgs {
     // Dispatch order, see work_index: the first `snake_rows` rows of `snake_len` workgroups each
     // are walked in alternating directions.  n_cus is host-side only (0: unknown).
     int snake_len, snake_rows;
+    // head_group > 0: an XCD works through its heads `head_group` at a time (all tiles of one
+    // group before the next group), so that the K / V of the heads in flight fit its L2
+    int head_group;
     int n_cus;
 };
 
@@ -270,13 +273,51 @@ __device__ __forceinline__ int work_index(const AttnArgs& a) {
             idx = row * a.snake_len + (a.snake_len / 8 - 1 - pos / 8) * 8 + (pos & 7);
         }
     }
+    if (a.head_group > 0) {
+        // Workgroup i runs on XCD i % 8.  Position j = i / 8 in that XCD's sequence takes, group
+        // after group of `head_group` heads (head = XCD + 8 * its index on the XCD), the tiles of
+        // the group heaviest first; the host checked batch * heads % 8 == 0.
+        const int n_bh = a.batch * a.heads;
+        const int xcd = idx & 7, j = idx >> 3;
+        const int per_xcd = n_bh >> 3;
+        const int n_levels = (int)gridDim.x / n_bh;
+        const int full = per_xcd / a.head_group;             // groups of full size
+        const int span = a.head_group * n_levels;            // workgroups per full group
+        int group = j / span, r = j - group * span, size = a.head_group;
+        if (group >= full) {                                 // the last, smaller group
+            group = full, r = j - full * span, size = per_xcd - full * a.head_group;
+        }
+        const int level = r / size, head = group * a.head_group + (r - level * size);
+        idx = level * n_bh + xcd + 8 * head;
+    }
     return idx;
 }
 // Host: `per_cu` workgroups of the kernel fit a CU at a time; rows that the grid does not fill
 // are left alone.
-inline void set_dispatch_order(AttnArgs* a, int64_t blocks, int per_cu) {
+inline void set_dispatch_order(AttnArgs* a, int64_t blocks, int per_cu, bool group_heads = false) {
     a->snake_len = a->n_cus & ~7;
     a->snake_rows = 0;
+    a->head_group = 0;
+    if (group_heads && a->n_cus >= 8) {
+        // K and V of one head against the L2 of an XCD (4 MB; three quarters of it budgeted).
+        // Heads are grouped only where a group fills the XCD's resident workgroups by itself (else
+        // several groups are in flight anyway) and the launch is at least four such fillings deep
+        // (a group's heavy workgroups start late; in a shallow launch they become its tail).
+        // Measured at bf16 B4 S2048 H32 D80 with a padding mask (groups of 4 of the 16 heads of an
+        // XCD): forward 162 -> 153 us, dQ 174 -> 163 us, dK/dV 222 -> 234 us (hence not there);
+        // without the two conditions: fp16 B8 S1024 H16 D64 forward 34 -> 42 us, bf16 B4 S2048 H16
+        // D128 forward 90 -> 100 us, S4096 306 -> 340 us.
+        const int64_t n_bh = (int64_t)a->batch * a->heads;
+        const int64_t head_bytes = 2 * (int64_t)a->sk * a->d * 2;
+        const int64_t fit = (3 << 20) / (head_bytes > 0 ? head_bytes : 1);
+        const int64_t levels = n_bh > 0 ? blocks / n_bh : 0;
+        const int64_t xcd_slots = (int64_t)(a->n_cus / 8) * per_cu;
+        if (n_bh % 8 == 0 && blocks % n_bh == 0 && fit >= 1 && fit < n_bh / 8 &&
+            fit * levels >= xcd_slots && blocks >= 4 * 8 * xcd_slots) {
+            a->head_group = (int)fit;
+            return;  // the order inside a group is heaviest first
+        }
+    }
     if (a->snake_len < 8 || !a->causal) return;
     const int64_t full_rows = blocks / a->snake_len;
     a->snake_rows = (int)(full_rows < per_cu ? full_rows : per_cu);
