@@ -194,6 +194,24 @@ def bench_epilogues(device, iters=40):
                                         "GBps": nbytes / sec / 1e9,
                                         "frac_of_hbm_peak": nbytes / sec / 1e9 / HBM_PEAK_GBS}
 
+    # backward of the bias-dropout(-residual) epilogue: dx = dropout mask applied to the upstream
+    # gradient (the mask is redrawn from seed and offset), dbias = its column sum
+    bws_bytes = lib.slapo_amd_colsum_workspace_bytes(T, Hd)
+    bws = torch.empty(bws_bytes // 4, dtype=torch.float32, device=device)
+    db1 = torch.empty(Hd, device=device, dtype=bf)
+
+    def dropres_bwd(i):  # reads the gradient (os_), writes dx (xs) and dbias
+        rc = lib.slapo_amd_bias_dropout_residual_bwd(P(os_[i]), P(xs[i]), P(db1), P(bws),
+                                                     bws_bytes, T, Hd, _lib.SLAPO_BF16, 0.1, 2013,
+                                                     0, ctypes.byref(plan), st)
+        assert rc == 0
+
+    sec = timed(dropres_bwd, n_rot)
+    nbytes = 2 * T * Hd * 2 + Hd * 2
+    out["bias_dropout_residual_bwd"] = {"bytes": nbytes, "us": sec * 1e6,
+                                        "GBps": nbytes / sec / 1e9,
+                                        "frac_of_hbm_peak": nbytes / sec / 1e9 / HBM_PEAK_GBS}
+
     # bias + dropout + residual + LayerNorm, training form: z, mean, rstd written for the backward
     zs = [torch.empty(T, Hd, device=device, dtype=bf) for _ in range(n_rot)]
     gam = torch.ones(Hd, device=device, dtype=bf)
@@ -325,6 +343,13 @@ def cpu_epilogue_baselines():
           lambda: OE.bias_gelu_back(gr, bi, y, torch.float32).to(bf))
     entry("bias_dropout_residual_fwd", 3 * T * Hd * e + Hd * e,
           lambda: OE.bias_dropout_residual(x, b1, res, 0.1, keep, torch.float32).to(bf))
+    gx = torch.randn(rows, Hd, generator=g).to(bf)
+
+    def dropres_bwd_cpu():
+        dx, dbias, _ = OE.bias_dropout_residual_bwd(gx, 0.1, keep, torch.float32)
+        return dx.to(bf), dbias.to(bf)
+
+    entry("bias_dropout_residual_bwd", 2 * T * Hd * e + Hd * e, dropres_bwd_cpu)
     entry("bias_dropout_residual_ln_fwd", 4 * T * Hd * e + 3 * Hd * e + 2 * T * 4,
           lambda: OE.bias_dropout_residual_layer_norm(x, b1, res, w, lb, 1e-5, 0.1, keep,
                                                       torch.float32)[0].to(bf))

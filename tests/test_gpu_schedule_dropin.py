@@ -228,3 +228,86 @@ def test_fork_rng_wraps_forward_and_decorrelates_ranks():
     # the fork leaves the default stream untouched (the draw came from the forked state)
     slapo_amd.set_random_seed(123, None, None, 0)
     assert outs[0][1] == torch.cuda.default_generators[0].get_offset()
+
+
+# ---- the attention wrappers of the other model schedules ---------------------------------------
+from oracle import attention as OA  # noqa: E402
+from tests import adapters as AD  # noqa: E402
+
+
+def _hf_padding_mask(b, s, valid, dtype):
+    """HF extended attention mask: 0 on valid keys, finfo.min on padded ones, [B,1,1,S]."""
+    m = torch.zeros(b, 1, 1, s, dtype=dtype, device="cuda")
+    for i, n in enumerate(valid):
+        m[i, :, :, n:] = torch.finfo(dtype).min
+    return m
+
+
+def _oracle_of(m, x, mask):
+    """What the wrapped FlashAttention computes, from its own weights, on the CPU in fp64."""
+    w = {n: p.detach().cpu().double() for n, p in m.named_parameters()}
+    b, s, _ = x.shape
+    h, d = m.num_attention_heads, m.attention_head_size
+    packed = x.cpu().double() @ w["qkv.weight"].t()
+    if "qkv.bias" in w:
+        packed = packed + w["qkv.bias"]
+    q, k, v = packed.view(b, s, h, 3 * d).split(d, dim=-1)
+    ctx = OA.xformers_ref(q, k, v, None if mask is None else mask.cpu().double(), m.output_proj,
+                          compute_dtype=torch.float64).reshape(b, s, h * d)
+    if m.output_proj:
+        ctx = ctx @ w["out_proj.weight"].t()
+        if "out_proj.bias" in w:
+            ctx = ctx + w["out_proj.bias"]
+    return ctx
+
+
+@pytest.mark.parametrize("family", ["gpt2", "gpt_neo", "opt", "bert", "albert"])
+def test_model_schedule_wrappers_call_and_trim_as_the_reference_does(family):
+    """Each wrapper is called the way its HF parent layer calls the original attention, and must
+    hand back what that layer unpacks: gpt2.py:241-264 and gpt_neo.py:193-215 (`outputs[:1]`),
+    opt.py:169-201 (`(out, None, None)`), bert.py:196-208 (`outputs[:1]`), albert.py:196-205
+    (`(context, None)`).  Values against the oracle at the bar of the reference's module test
+    (tests/test_op.py: atol = rtol = 5e-2 in fp16)."""
+    _seed(4)
+    dtype = torch.float16
+    cfg = AD.model_config()
+    wrapper = AD.make_adapter(family, op.FlashAttention, cfg, "cuda").to(dtype).cuda()
+    b, s = 2, 192
+    x = torch.randn(b, s, cfg.hidden_size, dtype=dtype, device="cuda")
+    mask = _hf_padding_mask(b, s, [s, 150], dtype)
+    if family == "gpt2":  # GPT2Block: attn(hidden, layer_past=, attention_mask=, head_mask=, ...)
+        out = wrapper(x, layer_past=None, attention_mask=mask, head_mask=None, use_cache=False,
+                      output_attentions=False)
+        assert isinstance(out, tuple) and len(out) == 1
+    elif family == "gpt_neo":  # GPTNeoBlock: same keywords without the encoder pair
+        out = wrapper(x, layer_past=None, attention_mask=mask, head_mask=None, use_cache=False,
+                      output_attentions=False)
+        assert isinstance(out, tuple) and len(out) == 1
+    elif family == "opt":  # OPTDecoderLayer unpacks three values
+        out = wrapper(hidden_states=x, past_key_value=None, attention_mask=mask,
+                      layer_head_mask=None, output_attentions=False)
+        assert len(out) == 3 and out[1] is None and out[2] is None
+    elif family == "bert":  # BertAttention: self(hidden, attention_mask, head_mask, ...)
+        out = wrapper(x, mask, None, None, None, None, False)
+        assert isinstance(out, tuple) and len(out) == 1
+    else:  # AlbertLayer: attention(hidden, attention_mask, head_mask, output_attentions)
+        out = wrapper(x, mask, None, False)
+        assert len(out) == 2 and out[1] is None
+    ref = _oracle_of(AD.inner(wrapper), x, mask)
+    torch.testing.assert_close(out[0].cpu().double(), ref, atol=5e-2, rtol=5e-2)
+
+
+def test_gpt_neo_wrapper_has_no_projection_biases_and_trains():
+    """bias=False (gpt_neo.py:171) removes the biases of qkv and out_proj; the block's tail then
+    runs as the two child calls (there is no bias for the fused pass to add)."""
+    _seed(5)
+    wrapper = AD.make_adapter("gpt_neo", op.FlashAttention,
+                              AD.model_config(resid_dropout=0.1, attention_dropout=0.1),
+                              "triton").half().cuda()
+    m = AD.inner(wrapper)
+    assert m.qkv.bias is None and m.out_proj.bias is None
+    x = torch.randn(2, 128, 256, dtype=torch.float16, device="cuda", requires_grad=True)
+    (out,) = wrapper(x, attention_mask=None)
+    out.float().sum().backward()
+    assert torch.isfinite(x.grad.float()).all() and m.qkv.weight.grad is not None
+    assert 0.05 < (out == 0).float().mean().item() < 0.15  # resid_dropout ran
