@@ -67,3 +67,61 @@ def test_static_scratch_rejects_sizes_beyond_the_array():
                                                None)
     assert rc == -7  # SLAPO_ERR_WORKSPACE
     assert b"workspace" in lib.slapo_amd_status_string(rc)
+
+
+def _static_call(dtype=torch.float16, b=2, s=256, h=4, d=64, seed=5):
+    lib = _lib.load()
+    g = torch.Generator().manual_seed(seed)
+    q, k, v, do = (torch.randn(b, s, h, d, generator=g).to(dtype).cuda() for _ in range(4))
+    o, lse, _ = K.attn_fwd(q, k, v, None, True, 0, d ** -0.5, 0.0, 0, 0, None)
+    prm = K.make_attn_params(q, k, v, o, None, True, 0, d ** -0.5, 0.0, 0, 0, None)
+    dq, dk, dv = torch.zeros_like(q), torch.zeros_like(k), torch.zeros_like(v)
+    strides = [K._bshd_strides(t) for t in (dq, dk, dv)]
+    keep = (q, k, v, do, o, lse, prm, strides)  # alive for as long as the closure is
+
+    def call():
+        rc = lib.slapo_amd_attn_bwd_static_scratch(
+            ctypes.byref(prm), _ptr(q), _ptr(k), _ptr(v), None, _ptr(o), _ptr(do), _ptr(lse),
+            _ptr(dq), _ptr(dk), _ptr(dv), *strides,
+            ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+        assert rc == 0, rc
+
+    return call, (dq, dk, dv), keep
+
+
+def test_static_scratch_call_leaves_device_memory_and_the_allocator_alone():
+    """The property the entry point exists for: between two points with no other work, neither
+    the device's free memory nor torch's allocator moves (no hipMalloc, no hipFree, no torch
+    allocation inside the call)."""
+    call, _, _keep = _static_call()
+    call()  # first call on the device: resolves the array's address, sets kernel attributes
+    torch.cuda.synchronize()
+    free0, _ = torch.cuda.mem_get_info()
+    alloc0, reserved0 = torch.cuda.memory_allocated(), torch.cuda.memory_reserved()
+    n_alloc0 = torch.cuda.memory_stats()["allocation.all.allocated"]
+    for _ in range(3):
+        call()
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free0
+    assert torch.cuda.memory_allocated() == alloc0 and torch.cuda.memory_reserved() == reserved0
+    assert torch.cuda.memory_stats()["allocation.all.allocated"] == n_alloc0
+
+
+def test_static_scratch_backward_under_graph_capture():
+    """After one call outside a capture (which resolves the array's address), the entry point can
+    be recorded into a HIP graph and replayed; every replay equals the eager result."""
+    call, grads, _keep = _static_call(torch.bfloat16, 1, 320, 2, 128, seed=6)
+    call()
+    torch.cuda.synchronize()
+    eager = [t.clone() for t in grads]
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        call()  # launches on the capturing stream
+    for round_ in range(3):
+        for t in grads:
+            t.zero_()  # eager work between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, want in zip(grads, eager):
+            assert torch.equal(got, want), f"replay {round_}"
