@@ -122,6 +122,27 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
     float m_run = -INFINITY;
     float m_ref = 0.f;  // what the exponentials subtract: m_run, or 0 while m_run is -inf
     float l_run = 0.f;  // this lane's share of the running sum
+    // kRefInMma: the matrix pipe subtracts the reference as well.  One more matrix instruction per
+    // tile whose A operand is a constant (kRefUnit in k-slot 0, zeros elsewhere) and whose B
+    // operand holds -m_ref / kRefUnit in that slot gives the start value of both score
+    // accumulators, so that the scores arrive relative to m_ref and a probability is one
+    // v_exp_f32.  The reference must then be a number of T: it is rounded to T when it moves (the
+    // row's probabilities and their sum share whatever value is subtracted, so the rounding
+    // cancels in the output, and the log-sum-exp is formed from the rounded value), kept within
+    // T's range (fp16: |m_ref| <= 60000 * 64 log2 units) and away from T's subnormals.
+    // Measured: 28 fewer vector instructions per tile (118 -> 90 at head_dim 64) change nothing at
+    // head_dim 64 (32.5 us either way at fp16 B8 S1024 H16 causal, 78.7 / 79.2 us with dropout),
+    // cost 3 % at head_dim 128 without dropout and 27 % in the window build that reads stored
+    // keep bits, and gain 9 % at head_dim 128 where the kernel draws its dropout bits (bf16 B4
+    // S2048 H16 causal, p 0.1: 209 -> 190 us): that build has the most live registers, and the
+    // subtractions' operands are what it no longer keeps.  Only that build uses it.  (Builds with
+    // a bias could not: the masking value -FLT_MAX is no number of T.)
+    constexpr bool kRefInMma = kBias == 0 && (kDrop == 1 || kDrop == 2) && kWin == 0 && DPAD > 96;
+    constexpr float kRefUnit = std::is_same<T, f16_t>::value ? 64.f : 1.f;
+    frag_t ones_frag, ref_frag;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) ones_frag[j] = (T)0.f, ref_frag[j] = (T)0.f;
+    if (g == 0) ones_frag[0] = (T)kRefUnit;
 
     const int wq_last = min(wq0 + 31, a.sq - 1);
     uint64_t drop_row_base = 0;
@@ -167,6 +188,7 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
     auto half_scores = [&](const T* kt, int kb, f32x16_t& s) __attribute__((always_inline)) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) s[r] = 0.f;
+        if constexpr (kRefInMma) s = Mma<T>::mma32(ones_frag, ref_frag, s);
 #pragma unroll
         for (int x = 0; x < DK; ++x)
             s = Mma<T>::mma32(lds_frag<T>(kt + kb * 32 * kPitch + k_off + 16 * x), qf[x], s);
@@ -236,19 +258,49 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
     // tile): only when the maximum exceeds it by more than kMaxSlack, so that the rescale of the
     // accumulators stays off the common path.  A row that has met nothing but masked keys
     // sits at -FLT_MAX and moves up to the first real key like any other.
-    auto update_reference = [&](float mx) __attribute__((always_inline)) {
-        const bool move = mx > m_run + kMaxSlack && mx != -INFINITY;
-        if (__builtin_expect(__builtin_amdgcn_ballot_w64(move) != 0, 0)) {
-            // exp2(old reference - new reference); an unset reference (-inf) scales by 0
-            const float alpha = (m_run == -INFINITY) ? 0.f : fast_exp2(m_run - mx);
-            if (move) {
-                m_run = mx;
-                m_ref = mx;
-                l_run *= alpha;
+    auto update_reference = [&](float mx, f32x16_t& s0, f32x16_t& s1)
+                                __attribute__((always_inline)) {
+        if constexpr (!kRefInMma) {
+            const bool move = mx > m_run + kMaxSlack && mx != -INFINITY;
+            if (__builtin_expect(__builtin_amdgcn_ballot_w64(move) != 0, 0)) {
+                // exp2(old reference - new reference); an unset reference (-inf) scales by 0
+                const float alpha = (m_run == -INFINITY) ? 0.f : fast_exp2(m_run - mx);
+                if (move) {
+                    m_run = mx;
+                    m_ref = mx;
+                    l_run *= alpha;
 #pragma unroll
-                for (int x = 0; x < DV; ++x)
+                    for (int x = 0; x < DV; ++x)
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) o_acc[x][r] *= alpha;
+                        for (int r = 0; r < 16; ++r) o_acc[x][r] *= alpha;
+                }
+            }
+        } else {
+            // mx is relative to m_ref here (the scores left the matrix pipe that way)
+            const bool move = (m_run == -INFINITY) ? mx != -INFINITY : mx > kMaxSlack;
+            if (__builtin_expect(__builtin_amdgcn_ballot_w64(move) != 0, 0)) {
+                // the new reference as a number of T (times kRefUnit), in range and normal
+                constexpr float kTop = std::is_same<T, f16_t>::value ? 60000.f : 3.0e38f;
+                constexpr float kTiny = std::is_same<T, f16_t>::value ? 6.2e-5f : 1.2e-38f;
+                float x = -(m_ref + mx) * (1.0f / kRefUnit);
+                x = fminf(fmaxf(x, -kTop), kTop);
+                if (fabsf(x) < kTiny) x = 0.f;
+                const T xt = (T)x;
+                const float m_new = -(float)xt * kRefUnit;
+                const float alpha = (m_run == -INFINITY) ? 0.f : fast_exp2(m_run - m_new);
+                if (move) {
+                    const float shift = m_new - m_ref;  // this tile's scores move with it
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) s0[r] -= shift, s1[r] -= shift;
+                    m_run = m_new;
+                    m_ref = m_new;
+                    if (g == 0) ref_frag[0] = xt;
+                    l_run *= alpha;
+#pragma unroll
+                    for (int x2 = 0; x2 < DV; ++x2)
+#pragma unroll
+                        for (int r = 0; r < 16; ++r) o_acc[x2][r] *= alpha;
+                }
             }
         }
     };
@@ -279,7 +331,7 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
     auto half_prob = [&](f32x16_t& s, int t, int kb, uint32_t (&pw)[8], uint32_t& drop_bits)
                          __attribute__((always_inline)) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) s[r] = fast_exp2(s[r] - m_ref);
+        for (int r = 0; r < 16; ++r) s[r] = fast_exp2(kRefInMma ? s[r] : s[r] - m_ref);
         if constexpr (kDrop != 0) {
             float psum = 0.f;
 #pragma unroll
@@ -337,7 +389,7 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
         half_scores(kt, 1, s1);
         const float mx =
             max_xor32(fmaxf(finish_half(s0, t, 0, mask_tag), finish_half(s1, t, 1, mask_tag)));
-        update_reference(mx);
+        update_reference(mx, s0, s1);
         half_prob(s0, t, 0, pw0, bits0);
         half_accumulate(vt, 0, pw0);
         half_prob(s1, t, 1, pw1, bits1);

@@ -205,13 +205,25 @@ __global__ __launch_bounds__(256) void bias_dropout_residual_fwd_kernel(
 // keeping per-thread fp32 column sums; the 4 row-lanes are combined through LDS and written
 // as one fp32 partial row per block.
 // ----------------------------------------------------------------------------------------
-constexpr int kRowsPerBlock = 64;
+constexpr int kRowsPerBlock = 64;  // at most; see colsum_rows_per_block
 constexpr int kRowLanes = 4;
 constexpr int kColLanes = 64;
 
+// Rows that one block walks: 64 where that still gives the device four blocks per CU or more,
+// else 32 or 16 (a block's rows run one after the other, so a narrow matrix in few blocks is
+// bound by latency: bf16 8192 x 1024 in 256 blocks of 64 rows took 15.7 us for 33.6 MB).  The
+// choice depends on the shape alone, so that the workspace size and the finishing kernel agree
+// with the launch.
+inline int colsum_rows_per_block(int64_t rows, int64_t cols) {
+    const int64_t col_blocks = (cols + 8 * kColLanes - 1) / (8 * kColLanes);
+    int rpb = kRowsPerBlock;
+    while (rpb > 16 && col_blocks * ((rows + rpb - 1) / rpb) < 1024) rpb /= 2;
+    return rpb;
+}
+
 template <typename T, int V, typename F>
 __device__ __forceinline__ void colsum_walk(int64_t rows, int64_t cols, float* __restrict__ partial,
-                                            bool want_sum, F&& body) {
+                                            bool want_sum, int rows_per_block, F&& body) {
     const int cx = threadIdx.x % kColLanes;
     const int ry = threadIdx.x / kColLanes;
     const int64_t chunk_col = (int64_t)blockIdx.x * kColLanes + cx;
@@ -220,10 +232,10 @@ __device__ __forceinline__ void colsum_walk(int64_t rows, int64_t cols, float* _
     float acc[V];
 #pragma unroll
     for (int i = 0; i < V; ++i) acc[i] = 0.f;
-    const int64_t r_begin = (int64_t)blockIdx.y * kRowsPerBlock;
+    const int64_t r_begin = (int64_t)blockIdx.y * rows_per_block;
     if (active) {
 #pragma unroll 4
-        for (int it = 0; it < kRowsPerBlock / kRowLanes; ++it) {
+        for (int it = 0; it < rows_per_block / kRowLanes; ++it) {
             const int64_t r = r_begin + ry + (int64_t)it * kRowLanes;
             if (r < rows) body(r, col0, acc);
         }
@@ -251,13 +263,13 @@ __global__ __launch_bounds__(256) void bias_gelu_bwd_kernel(const T* __restrict_
                                                             T* __restrict__ dx,
                                                             float* __restrict__ partial,
                                                             int64_t rows, int64_t cols,
-                                                            int want_sum) {
+                                                            int want_sum, int rows_per_block) {
     Chunk<T, V> b;
     {
         const int64_t col0 = ((int64_t)blockIdx.x * kColLanes + threadIdx.x % kColLanes) * V;
         if (col0 < cols) b = load_chunk_cached<T, V>(bias + col0);
     }
-    colsum_walk<T, V>(rows, cols, partial, want_sum != 0,
+    colsum_walk<T, V>(rows, cols, partial, want_sum != 0, rows_per_block,
                       [&](int64_t r, int64_t col0, float* acc) {
                           const int64_t off = r * cols + col0;
                           const Chunk<T, V> g = load_chunk<T, V>(grad + off);
@@ -281,8 +293,9 @@ __global__ __launch_bounds__(256) void bias_dropout_bwd_kernel(const T* __restri
                                                                float* __restrict__ partial,
                                                                int64_t rows, int64_t cols,
                                                                int want_sum, int write_dx,
+                                                               int rows_per_block,
                                                                DropoutState s) {
-    colsum_walk<T, V>(rows, cols, partial, want_sum != 0,
+    colsum_walk<T, V>(rows, cols, partial, want_sum != 0, rows_per_block,
                       [&](int64_t r, int64_t col0, float* acc) {
                           const int64_t off = r * cols + col0;
                           const Chunk<T, V> g = load_chunk<T, V>(grad + off);
@@ -795,7 +808,8 @@ int dropres_fwd_launch(const void* x, const void* bias, const void* residual, vo
 inline bool bwd_grid(int64_t rows, int64_t cols, int v, dim3* grid) {
     const int64_t chunk_cols = (cols + v - 1) / v;
     const int64_t gx = (chunk_cols + kColLanes - 1) / kColLanes;
-    const int64_t gy = (rows + kRowsPerBlock - 1) / kRowsPerBlock;
+    const int rpb = colsum_rows_per_block(rows, cols);
+    const int64_t gy = (rows + rpb - 1) / rpb;
     if (gx > 0x7FFFFFFF || gy > 65535) return false;
     *grid = dim3((unsigned)gx, (unsigned)gy);
     return true;
@@ -803,7 +817,8 @@ inline bool bwd_grid(int64_t rows, int64_t cols, int v, dim3* grid) {
 
 template <typename T>
 int finish_colsum(const float* partial, void* dbias, int64_t rows, int64_t cols, hipStream_t st) {
-    const int64_t n_partials = (rows + kRowsPerBlock - 1) / kRowsPerBlock;
+    const int rpb = colsum_rows_per_block(rows, cols);
+    const int64_t n_partials = (rows + rpb - 1) / rpb;
     const unsigned blocks = (unsigned)((cols + kFinCols - 1) / kFinCols);
     hipLaunchKernelGGL((colsum_finish_kernel<T>), dim3(blocks), dim3(256), 0, st, partial,
                        (T*)dbias, n_partials, cols);
@@ -819,11 +834,13 @@ int gelu_bwd_dispatch(const void* grad, const void* y, const void* bias, void* d
         constexpr int V = Elem<T>::kPerVec;
         if (!bwd_grid(rows, cols, V, &grid)) return SLAPO_ERR_SHAPE;
         hipLaunchKernelGGL((bias_gelu_bwd_kernel<T, V>), grid, dim3(256), 0, st, (const T*)grad,
-                           (const T*)y, (const T*)bias, (T*)dx, (float*)ws, rows, cols, want);
+                           (const T*)y, (const T*)bias, (T*)dx, (float*)ws, rows, cols, want,
+                           colsum_rows_per_block(rows, cols));
     } else {
         if (!bwd_grid(rows, cols, 1, &grid)) return SLAPO_ERR_SHAPE;
         hipLaunchKernelGGL((bias_gelu_bwd_kernel<T, 1>), grid, dim3(256), 0, st, (const T*)grad,
-                           (const T*)y, (const T*)bias, (T*)dx, (float*)ws, rows, cols, want);
+                           (const T*)y, (const T*)bias, (T*)dx, (float*)ws, rows, cols, want,
+                           colsum_rows_per_block(rows, cols));
     }
     int rc = check_launch();
     if (rc != SLAPO_OK || !dbias) return rc;
@@ -838,7 +855,8 @@ int dropres_bwd_launch(const void* grad, void* dx, void* ws, int64_t rows, int64
     const int write_dx = dx ? 1 : 0;
 #define SLAPO_LAUNCH_DB(MODE)                                                                  \
     hipLaunchKernelGGL((bias_dropout_bwd_kernel<T, V, MODE>), grid, dim3(256), 0, st,          \
-                       (const T*)grad, (T*)dx, (float*)ws, rows, cols, want, write_dx, s)
+                       (const T*)grad, (T*)dx, (float*)ws, rows, cols, want, write_dx,            \
+                       colsum_rows_per_block(rows, cols), s)
     const int mode = !dropout ? 0 : (V % 4 == 0 && s.g_shift >= 0 && s.t_shift >= 0) ? 1 : 2;
     if (mode == 0) SLAPO_LAUNCH_DB(0);
     if constexpr (V % 4 == 0) {
@@ -986,7 +1004,8 @@ inline bool dims_ok(int64_t rows, int64_t cols) {
 
 extern "C" size_t slapo_amd_colsum_workspace_bytes(int64_t rows, int64_t cols) {
     if (rows <= 0 || cols <= 0) return 0;
-    const int64_t n_partials = (rows + kRowsPerBlock - 1) / kRowsPerBlock;
+    const int rpb = colsum_rows_per_block(rows, cols);
+    const int64_t n_partials = (rows + rpb - 1) / rpb;
     return (size_t)n_partials * (size_t)cols * sizeof(float);
 }
 
