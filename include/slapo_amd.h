@@ -236,7 +236,9 @@ size_t slapo_amd_attn_keep_mask_bytes(const slapo_attn_params* prm);
  * values at or below -5e8 (other than -inf) are one masking value; a query row that sees nothing
  * but keys masked with it attends to them uniformly, as in the reference's arithmetic, and its
  * lse slot holds n * 2^100 (n = number of those keys) for the backward, which gives such rows the
- * gradients of that uniform softmax. */
+ * gradients of that uniform softmax.  The backward must therefore be given the same bias as the
+ * forward: only its bias builds decode that value (the host cannot inspect lse, so a backward
+ * called without the bias returns zero gradients for such rows without an error). */
 int slapo_amd_attn_fwd(const slapo_attn_params* prm, const void* q, const void* k, const void* v,
                        const float* bias, void* o, float* lse, void* stream);
 
