@@ -67,6 +67,21 @@ def _make_inputs(cfg, device):
     return [torch.randn(shape, generator=g).to(torch.float16).to(device) for _ in range(4)]
 
 
+SETTLE_SECONDS = 0.03
+
+
+def _settle(fn):
+    """Runs fn back to back for SETTLE_SECONDS of wall time before a timed measurement: a few
+    launches are not enough for the device clock to settle after an idle stretch (the first
+    10-20 ms of a burst run 5-15 % slow on these boxes).  `--settle-ms 0` switches it off, for
+    counter collection, where every dispatch is recorded."""
+    t_end = time.perf_counter() + SETTLE_SECONDS
+    while time.perf_counter() < t_end:
+        for _ in range(8):
+            fn()
+    torch.cuda.synchronize()
+
+
 class AttentionStep:
     """Forward + backward of the attention op through the C ABI on preallocated buffers."""
 
@@ -136,7 +151,7 @@ def bench_epilogues(device, iters=40):
     def timed(fn, n_rot):
         for i in range(n_rot):
             fn(i)
-        torch.cuda.synchronize()
+        _settle(lambda: fn(0))
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         for i in range(iters):
@@ -521,7 +536,7 @@ def bench_other_attention(device, iters=20, with_cpu=True):
         def timed(fn):
             for _ in range(3):
                 fn()
-            torch.cuda.synchronize()
+            _settle(fn)
             e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             e0.record()
             for _ in range(iters):
@@ -559,6 +574,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--repeats", type=int, default=25,
                     help="timed loops of --steps steps; the median loop is reported")
+    ap.add_argument("--settle-ms", type=float, default=30.0,
+                    help="back-to-back launches for this long before each timed sub-benchmark")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-epilogues", action="store_true")
     ap.add_argument("--no-other-attention", action="store_true",
@@ -573,6 +590,8 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py needs an MI355X (no GPU visible)")
 
+    global SETTLE_SECONDS
+    SETTLE_SECONDS = max(args.settle_ms, 0.0) * 1e-3
     cfg = WORKLOAD
     device = torch.device("cuda", 0)
     torch.cuda.set_device(device)
