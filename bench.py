@@ -49,8 +49,8 @@ FP32_VECTOR_PEAK_TFLOPS = 157.3
 # HBM bytes per launch of the dK/dV kernel on WORKLOAD, from rocprofv3 --pmc FETCH_SIZE and
 # WRITE_SIZE (KiB per dispatch), each scaled by the same counter's reading for a 256 MiB copy
 # (FETCH_SIZE reads half the copied bytes: factor 2.0; WRITE_SIZE factor 1.0):
-# (43.23e3 * 2.0 + 32.77e3) KiB = 122 MB against 101.7 MB algorithmic.  Summary under profiles/.
-DKDV_TRAFFIC_BYTES = (43.23e3 * 2.0 + 32.77e3) * 1024
+# (43.93e3 * 2.0 + 32.77e3) KiB = 123.5 MB against 101.7 MB algorithmic.  Summary under profiles/.
+DKDV_TRAFFIC_BYTES = (43.93e3 * 2.0 + 32.77e3) * 1024
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 
 WORKLOAD = dict(name="gpt2-medium causal attention fwd+bwd", dtype="fp16", batch=8, seq=1024,
