@@ -1,5 +1,5 @@
-"""The reference-side binding that INTEGRATION.md shows (the code a maintainer would paste into
-slapo/op/attention.py) is executed here exactly as documented.
+"""The reference-side binding shown in the integration guide at the repository root (the code a
+maintainer would paste into slapo/op/attention.py) is executed here exactly as documented.
 
 CPU: its ctypes structs are compared, field by field, with what the C compiler makes of
 include/slapo_amd.h (offsets and sizes printed by a small program built with gcc), and so is the
@@ -25,7 +25,7 @@ HEADER_DIR = os.path.join(ROOT, "include")
 def _stub_source():
     text = open(DOC).read()
     m = re.search(r"<!-- stub:begin -->\s*```python\n(.*?)```\s*<!-- stub:end -->", text, re.S)
-    assert m, "INTEGRATION.md lost its stub markers"
+    assert m, "the integration guide lost its stub markers"
     return m.group(1)
 
 
@@ -91,7 +91,7 @@ def test_stub_prototypes_agree_with_the_package_table(stub):
 
 
 class _Op(torch.nn.Module):
-    """FlashAttentionOp reduced to the two edits INTEGRATION.md asks for: the registry branch sets
+    """FlashAttentionOp reduced to the two edits that the guide asks for: the registry branch sets
     pkg / attn_fn, the forward takes the new first branch."""
 
     def __init__(self, attn_fn, apply_causal_mask, scale=None):
