@@ -224,7 +224,9 @@ typedef struct slapo_attn_params {
      * the same stream draws them and the forward kernel reads them), and a backward that is given
      * the same buffer reads them instead of drawing every Philox block again in both of its
      * kernels.  The results are bitwise the same with and without it.  Words whose keys no query
-     * of the row's 32-query group can see under the causal mask or the window are not written.  Layout: uint32 words [batch*heads][ceil(seqlen_k/32)][pitch],
+     * of the row's 32-query group can see under the causal mask are not written; with a window,
+     * only the words that hold a key the row itself can see are (the rest is never applied to a
+     * non-zero probability).  Layout: uint32 words [batch*heads][ceil(seqlen_k/32)][pitch],
      * pitch = seqlen_q rounded up to 4; bit j of word (bh, w, i) = keep(query i, key 32 w + j). */
     void* keep_mask;
 } slapo_attn_params;

@@ -71,18 +71,23 @@ __global__ __launch_bounds__(256) void attn_delta_scalar_kernel(const AttnArgs a
 // query i and stores them as one word, keep_mask[(bh * mask_words + w) * mask_pitch + i], bit j =
 // keep(i, 32 w + j).  The matrix kernels then only test bits; drawing inside the forward kernel
 // costs about forty vector-ALU cycles per score beside thirty-two (head_dim 128) or sixteen (64)
-// of matrix work.  Words whose 64-key tile no query of the row's 32-query group can see (causal
-// mask, local window) are never read and are left unwritten.
+// of matrix work.  Only words that hold a key the row itself can see are drawn: the kernels read
+// whole words of every 64-key tile that some query of a 32-query group sees, but a bit that
+// belongs to a pair outside the row's own mask meets a probability of zero, so what such words
+// hold does not matter and they are left as they are.  With a local window the grid's second
+// dimension counts words from the first one of the row's window (window / 32 + 1 of them, not
+// seqlen_k / 32: every thread then has a word to draw); without one it is the word itself.
 // kExact: any launch geometry of the dropout plan and any seqlen_k (one Philox block per bit).
 template <bool kExact>
 __global__ __launch_bounds__(256) void keep_mask_kernel(const AttnArgs a) {
     const int i = blockIdx.x * 256 + threadIdx.x;
-    const int w = blockIdx.y;
     const int bh = blockIdx.z;
     if (i >= a.sq) return;
-    const int tile0 = (w >> 1) * 64, grp0 = i & ~31;
-    if (a.causal && tile0 > grp0 + 31) return;
-    if (a.window > 0 && grp0 - (tile0 + 63) >= a.window) return;
+    int w = blockIdx.y;
+    if (a.window > 0) w += max(i - a.window + 1, 0) >> 5;
+    if (w >= a.mask_words) return;
+    if (a.causal && 32 * w > i) return;
+    if (a.window > 0 && i - (32 * w + 31) >= a.window) return;
     const uint64_t row_base = ((uint64_t)bh * a.sq + (uint64_t)i) * (uint64_t)a.sk;
     uint32_t word = 0;
 #pragma unroll
@@ -106,7 +111,9 @@ bool keep_mask_kernel_fits(const AttnArgs& a) {
 int draw_keep_mask(const AttnArgs& a, hipStream_t st) {
     const int64_t bh = (int64_t)a.batch * a.heads;
     if (!keep_mask_kernel_fits(a)) return SLAPO_ERR_SHAPE;
-    const dim3 grid((unsigned)((a.sq + 255) / 256), (unsigned)a.mask_words, (unsigned)bh);
+    // with a window: the words of a row's own window (it spans window / 32 + 1 words at most)
+    const int words = a.window > 0 ? min(a.mask_words, a.window / 32 + 2) : a.mask_words;
+    const dim3 grid((unsigned)((a.sq + 255) / 256), (unsigned)words, (unsigned)bh);
     if (a.dropout == 1)
         hipLaunchKernelGGL(keep_mask_kernel<false>, grid, dim3(256), 0, st, a);
     else

@@ -304,10 +304,10 @@ def test_dropout_keep_bits_saved_by_the_forward(dtype, shape, causal, window, ma
     keep = _torch_keep(b, h, s, s, p)
     i, j = torch.arange(s)[:, None], torch.arange(s)[None, :]
     visited = torch.ones(s, s, dtype=torch.bool)
-    if causal:   # the forward skips 64-key tiles above the diagonal of each 32-query group
+    if window:   # drawn ahead of the forward: the 32-key words that hold a key the row itself sees
+        visited &= ((j // 32) * 32 <= i) & (i - ((j // 32) * 32 + 31) < window)
+    elif causal:  # the forward skips 64-key tiles above the diagonal of each 32-query group
         visited &= (j // 64) * 64 <= (i // 32) * 32 + 31
-    if window:   # ... and those wholly outside the window of the group
-        visited &= (i // 32) * 32 - ((j // 64) * 64 + 63) < window
     if not masked:
         assert torch.equal(got[:, visited], keep[:, visited])
     else:  # skipped padded tiles differ per batch: check the unpadded prefix of each batch
@@ -549,12 +549,14 @@ def test_full_size_cfg5_properties(window):
     packed = (keep.view(b * h, s, n_words, 32).to(torch.int64) * weights).sum(-1)  # [bh, i, w]
     packed = packed.permute(0, 2, 1)                                                # [bh, w, i]
     w = torch.arange(n_words, device="cuda")
-    # a 32-key word is written iff its 64-key tile is visited by the 32-query group of the row
+    # without a window (bits drawn by the forward) a 32-key word is written iff its 64-key tile is
+    # visited by the 32-query group of the row; with one (bits drawn ahead of the forward) iff it
+    # holds a key that the row itself sees
     tile0 = (w[:, None] // 2) * 64
     grp0 = (i[None, :] // 32) * 32
     visited = tile0 <= grp0 + 31
     if window:
-        visited &= grp0 - (tile0 + 63) < window
+        visited = (32 * w[:, None] <= i[None, :]) & (i[None, :] - (32 * w[:, None] + 31) < window)
     assert torch.equal(words[:, visited], packed[:, visited])
     del keep, packed, words
 
