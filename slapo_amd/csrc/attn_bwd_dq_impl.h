@@ -40,14 +40,16 @@ constexpr int kVRing = 2;
 // kBias: 0 = no additive bias, 1 = any layout (read from memory per score), 2 = the bias depends on
 // the key only (stride 0 over the queries): its 64 values per key tile travel through LDS beside
 // the K / V tile, and the tile bodies have neither global loads nor branches for them.
-template <typename T, int DPAD, int kBias, int kDrop, bool kStagger>
+template <typename T, int DPAD, int kBias, int kDrop, bool kStagger, int kSteps>
 __global__ __launch_bounds__(kThreads, (kStagger && DPAD > 64 ? 1 : 2)) void attn_bwd_dq_kernel(
     const AttnArgs a) {
     typedef typename Mma<T>::frag frag_t;
     typedef TileStage<T, DPAD, kBN, kThreads> Stage;
     constexpr int kPitch = Stage::kPitch;
     constexpr int kTileElems = kBN * kPitch;
-    constexpr int DK = DPAD / 16;  // k-steps over the head dimension
+    // k-steps over the head dimension: DPAD / 16, or one fewer where the launcher guarantees
+    // head_dim <= 16 * kSteps (head_dim 80 in the 96-wide build)
+    constexpr int DK = kSteps;
     constexpr int DV = DPAD / 32;  // 32-row blocks of dQ^T
 
     extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -512,7 +514,7 @@ __global__ __launch_bounds__(kThreads, (kStagger && DPAD > 64 ? 1 : 2)) void att
     }
 }
 
-template <typename T, int DPAD, int kBias, int kDrop, bool kStagger>
+template <typename T, int DPAD, int kBias, int kDrop, bool kStagger, int kSteps>
 int launch(const AttnArgs& a, hipStream_t st) {
     typedef TileStage<T, DPAD, kBN, kThreads> Stage;
     const size_t smem = (size_t)(kKRing + kVRing) * kBN * Stage::kPitch * sizeof(T) +
@@ -520,39 +522,40 @@ int launch(const AttnArgs& a, hipStream_t st) {
     const int n_qt = (a.sq + kBM - 1) / kBM;
     const int64_t blocks = (int64_t)n_qt * a.batch * a.heads;
     if (blocks <= 0 || blocks > 0x7FFFFFFF) return SLAPO_ERR_SHAPE;
-    auto kern = attn_bwd_dq_kernel<T, DPAD, kBias, kDrop, kStagger>;
+    auto kern = attn_bwd_dq_kernel<T, DPAD, kBias, kDrop, kStagger, kSteps>;
     static std::atomic<uint64_t> lds_ready{0};  // per instantiation, one bit per device
     if (allow_dynamic_lds(reinterpret_cast<const void*>(kern), smem, lds_ready) != SLAPO_OK)
         return SLAPO_ERR_LAUNCH;
     AttnArgs ordered = a;
-    set_dispatch_order(&ordered, blocks, (kStagger && DPAD > 64) ? 1 : 2, true);
+    set_dispatch_order(&ordered, blocks, (kStagger && DPAD > 64) ? 1 : 2);
     hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kThreads), smem, st, ordered);
     return check_launch();
 }
 
-template <typename T, int DPAD, bool kStagger>
+template <typename T, int DPAD, bool kStagger, int kSteps = DPAD / 16>
 int dispatch_flags(const AttnArgs& a, hipStream_t st) {
     if (a.has_bias) {
         if (a.bs[2] == 0) {  // the bias depends on the key only
-            if (a.dropout == 1) return launch<T, DPAD, 2, 1, kStagger>(a, st);
-            if (a.dropout == 2) return launch<T, DPAD, 2, 2, kStagger>(a, st);
-            if (a.dropout == 3) return launch<T, DPAD, 2, 3, kStagger>(a, st);
-            return launch<T, DPAD, 2, 0, kStagger>(a, st);
+            if (a.dropout == 1) return launch<T, DPAD, 2, 1, kStagger, kSteps>(a, st);
+            if (a.dropout == 2) return launch<T, DPAD, 2, 2, kStagger, kSteps>(a, st);
+            if (a.dropout == 3) return launch<T, DPAD, 2, 3, kStagger, kSteps>(a, st);
+            return launch<T, DPAD, 2, 0, kStagger, kSteps>(a, st);
         }
-        if (a.dropout == 1) return launch<T, DPAD, 1, 1, kStagger>(a, st);
-        if (a.dropout == 2) return launch<T, DPAD, 1, 2, kStagger>(a, st);
-        if (a.dropout == 3) return launch<T, DPAD, 1, 3, kStagger>(a, st);
-        return launch<T, DPAD, 1, 0, kStagger>(a, st);
+        if (a.dropout == 1) return launch<T, DPAD, 1, 1, kStagger, kSteps>(a, st);
+        if (a.dropout == 2) return launch<T, DPAD, 1, 2, kStagger, kSteps>(a, st);
+        if (a.dropout == 3) return launch<T, DPAD, 1, 3, kStagger, kSteps>(a, st);
+        return launch<T, DPAD, 1, 0, kStagger, kSteps>(a, st);
     }
-    if (a.dropout == 1) return launch<T, DPAD, 0, 1, kStagger>(a, st);
-    if (a.dropout == 2) return launch<T, DPAD, 0, 2, kStagger>(a, st);
-    if (a.dropout == 3) return launch<T, DPAD, 0, 3, kStagger>(a, st);
-    return launch<T, DPAD, 0, 0, kStagger>(a, st);
+    if (a.dropout == 1) return launch<T, DPAD, 0, 1, kStagger, kSteps>(a, st);
+    if (a.dropout == 2) return launch<T, DPAD, 0, 2, kStagger, kSteps>(a, st);
+    if (a.dropout == 3) return launch<T, DPAD, 0, 3, kStagger, kSteps>(a, st);
+    return launch<T, DPAD, 0, 0, kStagger, kSteps>(a, st);
 }
 
 template <typename T>
 int dispatch(const AttnArgs& a, hipStream_t st) {
     if (a.d <= 64) return dispatch_flags<T, 64, true>(a, st);
+    if (a.d <= 80) return dispatch_flags<T, 96, false, 5>(a, st);  // five k-steps cover head_dim 80
     if (a.d <= 96) return dispatch_flags<T, 96, false>(a, st);
     if (a.d <= 128) {
         // a local window leaves mostly masked tiles, whose bodies spill at two workgroups per CU;

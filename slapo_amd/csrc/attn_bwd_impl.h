@@ -54,7 +54,7 @@ constexpr bool bwd_two_per_cu(int dpad, int drop, int kb) {
 // KB = blocks of 32 keys per wavefront.  KB = 2 halves the LDS operand traffic per matrix
 // instruction (every Q / dO fragment read feeds two MFMAs) at the price of twice the resident
 // fragments and accumulators, i.e. one wavefront per SIMD instead of two.
-template <typename T, int DPAD, int kBias, int kDrop, int KB>
+template <typename T, int DPAD, int kBias, int kDrop, int KB, int kSteps>
 // Two workgroups per CU up to DPAD 96, one at 128 (192 resident accumulator / fragment registers)
 // and at 96 with the forward's keep bits (measured 23-35 % slower with two than with one).
 __global__ __launch_bounds__(kBwdThreads, (bwd_two_per_cu(DPAD, kDrop, KB) ? 2 : 1)) void attn_bwd_kernel(
@@ -64,7 +64,9 @@ __global__ __launch_bounds__(kBwdThreads, (bwd_two_per_cu(DPAD, kDrop, KB) ? 2 :
     typedef BwdSmem<T, DPAD> SM;
     typedef typename SM::QStage QStage;
     constexpr int kPitch = SM::kPitch;
-    constexpr int DK = DPAD / 16;          // k-steps over head dim
+    // k-steps over the head dimension: DPAD / 16, or one fewer where the launcher guarantees
+    // head_dim <= 16 * kSteps (head_dim 80 in the 96-wide build)
+    constexpr int DK = kSteps;
     constexpr int DV = DPAD / 32;          // 32-row blocks of dK^T / dV^T
     constexpr int kWaveKeys = 32 * KB;
     constexpr int kBN = kBwdWaves * kWaveKeys;  // keys per workgroup
@@ -628,7 +630,7 @@ __global__ __launch_bounds__(kBwdThreads, (bwd_two_per_cu(DPAD, kDrop, KB) ? 2 :
     }
 }
 
-template <typename T, int DPAD, int kBias, int kDrop, int KB>
+template <typename T, int DPAD, int kBias, int kDrop, int KB, int kSteps>
 int launch(const AttnArgs& a, hipStream_t st) {
     typedef BwdSmem<T, DPAD> SM;
     const size_t smem = SM::kBytes;
@@ -636,7 +638,7 @@ int launch(const AttnArgs& a, hipStream_t st) {
     const int n_kt = (a.sk + kBN - 1) / kBN;
     const int64_t blocks = (int64_t)n_kt * a.batch * a.heads;
     if (blocks <= 0 || blocks > 0x7FFFFFFF) return SLAPO_ERR_SHAPE;
-    auto kern = attn_bwd_kernel<T, DPAD, kBias, kDrop, KB>;
+    auto kern = attn_bwd_kernel<T, DPAD, kBias, kDrop, KB, kSteps>;
     static std::atomic<uint64_t> lds_ready{0};  // per instantiation, one bit per device
     if (allow_dynamic_lds(reinterpret_cast<const void*>(kern), smem, lds_ready) != SLAPO_OK)
         return SLAPO_ERR_LAUNCH;
@@ -649,28 +651,30 @@ int launch(const AttnArgs& a, hipStream_t st) {
 // Two key blocks per wavefront (KB = 2, one wavefront per SIMD) measured slower than KB = 1 with two
 // wavefronts per SIMD on MI355X (92 us against 70 us at fp16 B8 S1024 H16 D64 causal): the second
 // resident wavefront hides more latency than the halved LDS traffic saves.  Only KB = 1 is built.
-template <typename T, int DPAD, int kBias, int kDrop>
+template <typename T, int DPAD, int kBias, int kDrop, int kSteps>
 int launch_kb(const AttnArgs& a, hipStream_t st) {
-    return launch<T, DPAD, kBias, kDrop, 1>(a, st);
+    return launch<T, DPAD, kBias, kDrop, 1, kSteps>(a, st);
 }
 
-template <typename T, int DPAD, int kBias>
+template <typename T, int DPAD, int kBias, int kSteps>
 int dispatch_drop(const AttnArgs& a, hipStream_t st) {
-    if (a.dropout == 1) return launch_kb<T, DPAD, kBias, 1>(a, st);
-    if (a.dropout == 2) return launch_kb<T, DPAD, kBias, 2>(a, st);
-    if (a.dropout == 3) return launch_kb<T, DPAD, kBias, 3>(a, st);
-    return launch_kb<T, DPAD, kBias, 0>(a, st);
+    if (a.dropout == 1) return launch_kb<T, DPAD, kBias, 1, kSteps>(a, st);
+    if (a.dropout == 2) return launch_kb<T, DPAD, kBias, 2, kSteps>(a, st);
+    if (a.dropout == 3) return launch_kb<T, DPAD, kBias, 3, kSteps>(a, st);
+    return launch_kb<T, DPAD, kBias, 0, kSteps>(a, st);
 }
 
-template <typename T, int DPAD>
+template <typename T, int DPAD, int kSteps = DPAD / 16>
 int dispatch_flags(const AttnArgs& a, hipStream_t st) {
-    if (!a.has_bias) return dispatch_drop<T, DPAD, 0>(a, st);
-    return a.bs[2] == 0 ? dispatch_drop<T, DPAD, 2>(a, st) : dispatch_drop<T, DPAD, 1>(a, st);
+    if (!a.has_bias) return dispatch_drop<T, DPAD, 0, kSteps>(a, st);
+    return a.bs[2] == 0 ? dispatch_drop<T, DPAD, 2, kSteps>(a, st)
+                        : dispatch_drop<T, DPAD, 1, kSteps>(a, st);
 }
 
 template <typename T>
 int dispatch(const AttnArgs& a, hipStream_t st) {
     if (a.d <= 64) return dispatch_flags<T, 64>(a, st);
+    if (a.d <= 80) return dispatch_flags<T, 96, 5>(a, st);  // five k-steps cover head_dim 80
     if (a.d <= 96) return dispatch_flags<T, 96>(a, st);
     if (a.d <= 128) return dispatch_flags<T, 128>(a, st);
     return SLAPO_ERR_SHAPE;

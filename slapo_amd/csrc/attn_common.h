@@ -303,10 +303,11 @@ inline void set_dispatch_order(AttnArgs* a, int64_t blocks, int per_cu, bool gro
         // Heads are grouped only where a group fills the XCD's resident workgroups by itself (else
         // several groups are in flight anyway) and the launch is at least four such fillings deep
         // (a group's heavy workgroups start late; in a shallow launch they become its tail).
-        // Measured at bf16 B4 S2048 H32 D80 with a padding mask (groups of 4 of the 16 heads of an
-        // XCD): forward 162 -> 153 us, dQ 174 -> 163 us, dK/dV 222 -> 234 us (hence not there);
-        // without the two conditions: fp16 B8 S1024 H16 D64 forward 34 -> 42 us, bf16 B4 S2048 H16
-        // D128 forward 90 -> 100 us, S4096 306 -> 340 us.
+        // Measured at bf16 B4 S2048 H32 D80 (groups of 4 of the 16 heads of an XCD), clocks
+        // settled: forward 132 -> 127 us with a padding mask, 146 -> 141 us without, 252 -> 236 us
+        // without the causal mask; dQ unchanged (163 us), dK/dV 222 -> 234 us: only the forward
+        // asks for it.  Without the two conditions: fp16 B8 S1024 H16 D64 forward 34 -> 42 us, bf16
+        // B4 S2048 H16 D128 forward 90 -> 100 us, S4096 306 -> 340 us.
         const int64_t n_bh = (int64_t)a->batch * a->heads;
         const int64_t head_bytes = 2 * (int64_t)a->sk * a->d * 2;
         const int64_t fit = (3 << 20) / (head_bytes > 0 ? head_bytes : 1);

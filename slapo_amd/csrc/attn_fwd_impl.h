@@ -32,7 +32,7 @@ constexpr int kBM = kWaves * 32;
 constexpr int kBN = 64;
 constexpr float kMaxSlack = 8.0f;  // hysteresis of the softmax reference, log2 units
 
-template <typename T, int DPAD, int kBias, int kDrop, int kWin>
+template <typename T, int DPAD, int kBias, int kDrop, int kWin, int kSteps>
 __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void attn_fwd_kernel(
     const AttnArgs a_in) {
     // kBias: 0 = no additive bias, 1 = any layout (read from memory per score), 2 = the bias
@@ -51,7 +51,9 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
     typedef TileStage<T, DPAD, kBN, kThreads> Stage;
     constexpr int kPitch = Stage::kPitch;
     constexpr int kTileElems = kBN * kPitch;
-    constexpr int DK = DPAD / 16;  // k-steps of S^T = K Q^T
+    // k-steps of S^T = K Q^T: DPAD / 16, or one fewer where the launcher guarantees head_dim <=
+    // 16 * kSteps (head_dim 80 in the 96-wide build: the sixth step would multiply zeros)
+    constexpr int DK = kSteps;
     constexpr int DV = DPAD / 32;  // 32-row blocks of O^T
 
     extern __shared__ __align__(16) unsigned char smem_raw[];
@@ -509,7 +511,7 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
     }
 }
 
-template <typename T, int DPAD, int kBias, int kDrop, int kWin>
+template <typename T, int DPAD, int kBias, int kDrop, int kWin, int kSteps>
 int launch(const AttnArgs& a, hipStream_t st) {
     typedef TileStage<T, DPAD, kBN, kThreads> Stage;
     const size_t smem = (size_t)4 * kBN * Stage::kPitch * sizeof(T) +
@@ -517,51 +519,56 @@ int launch(const AttnArgs& a, hipStream_t st) {
     const int n_qt = (a.sq + kBM - 1) / kBM;
     const int64_t blocks = (int64_t)n_qt * a.batch * a.heads;
     if (blocks <= 0 || blocks > 0x7FFFFFFF) return SLAPO_ERR_SHAPE;
-    auto kern = attn_fwd_kernel<T, DPAD, kBias, kDrop, kWin>;
+    auto kern = attn_fwd_kernel<T, DPAD, kBias, kDrop, kWin, kSteps>;
     static std::atomic<uint64_t> lds_ready{0};  // per instantiation, one bit per device
     if (allow_dynamic_lds(reinterpret_cast<const void*>(kern), smem, lds_ready) != SLAPO_OK)
         return SLAPO_ERR_LAUNCH;
     AttnArgs ordered = a;
-    set_dispatch_order(&ordered, blocks, (DPAD <= 64 && kDrop == 0) ? 3 : 2, true);
+    // (head groups: not where the kernel draws or applies dropout bits -- its workgroups run twice as
+    // long there and a group's late heavy ones become the tail: 314 -> 350 us at bf16 B4 S2048 H32
+    // D80 causal, p 0.1, 588 -> 667 us at fp16 B2 S4096 H32 D96)
+    set_dispatch_order(&ordered, blocks, (DPAD <= 64 && kDrop == 0) ? 3 : 2, kDrop == 0);
     hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kThreads), smem, st, ordered);
     return check_launch();
 }
 
-template <typename T, int DPAD, int kWin>
+template <typename T, int DPAD, int kWin, int kSteps>
 int dispatch_nobias(const AttnArgs& a, hipStream_t st) {
-    if (a.dropout == 1) return launch<T, DPAD, 0, 1, kWin>(a, st);
-    if (a.dropout == 2) return launch<T, DPAD, 0, 2, kWin>(a, st);
+    if (a.dropout == 1) return launch<T, DPAD, 0, 1, kWin, kSteps>(a, st);
+    if (a.dropout == 2) return launch<T, DPAD, 0, 2, kWin, kSteps>(a, st);
     if (a.dropout == 3) {  // stored keep bits: local-window calls only, see attn_capi.hip
         if constexpr (kWin != 0)
-            return launch<T, DPAD, 0, 3, kWin>(a, st);
+            return launch<T, DPAD, 0, 3, kWin, kSteps>(a, st);
         else
             return SLAPO_ERR_ARG;
     }
-    return launch<T, DPAD, 0, 0, kWin>(a, st);
+    return launch<T, DPAD, 0, 0, kWin, kSteps>(a, st);
 }
-template <typename T, int DPAD>
+template <typename T, int DPAD, int kSteps = DPAD / 16>
 int dispatch_flags(const AttnArgs& a, hipStream_t st) {
     if (a.has_bias) {
         // one build for both: with a bias the window-free build measured slower (it spills more
         // at head_dim 64 and 96: 266 against 185 us at bf16 B4 S2048 H32 D80 with a padding mask)
         if (a.bs[2] == 0) {  // the bias depends on the key only
-            if (a.dropout == 1) return launch<T, DPAD, 2, 1, 2>(a, st);
-            if (a.dropout == 2) return launch<T, DPAD, 2, 2, 2>(a, st);
-            if (a.dropout == 3) return launch<T, DPAD, 2, 3, 2>(a, st);
-            if (a.window <= 0) return launch<T, DPAD, 2, 0, 0>(a, st);
-            return launch<T, DPAD, 2, 0, 2>(a, st);
+            if (a.dropout == 1) return launch<T, DPAD, 2, 1, 2, kSteps>(a, st);
+            if (a.dropout == 2) return launch<T, DPAD, 2, 2, 2, kSteps>(a, st);
+            if (a.dropout == 3) return launch<T, DPAD, 2, 3, 2, kSteps>(a, st);
+            if (a.window <= 0) return launch<T, DPAD, 2, 0, 0, kSteps>(a, st);
+            return launch<T, DPAD, 2, 0, 2, kSteps>(a, st);
         }
-        if (a.dropout == 1) return launch<T, DPAD, 1, 1, 2>(a, st);
-        if (a.dropout == 2) return launch<T, DPAD, 1, 2, 2>(a, st);
-        if (a.dropout == 3) return launch<T, DPAD, 1, 3, 2>(a, st);
-        return launch<T, DPAD, 1, 0, 2>(a, st);
+        if (a.dropout == 1) return launch<T, DPAD, 1, 1, 2, kSteps>(a, st);
+        if (a.dropout == 2) return launch<T, DPAD, 1, 2, 2, kSteps>(a, st);
+        if (a.dropout == 3) return launch<T, DPAD, 1, 3, 2, kSteps>(a, st);
+        return launch<T, DPAD, 1, 0, 2, kSteps>(a, st);
     }
-    return a.window > 0 ? dispatch_nobias<T, DPAD, 1>(a, st) : dispatch_nobias<T, DPAD, 0>(a, st);
+    return a.window > 0 ? dispatch_nobias<T, DPAD, 1, kSteps>(a, st)
+                        : dispatch_nobias<T, DPAD, 0, kSteps>(a, st);
 }
 
 template <typename T>
 int dispatch(const AttnArgs& a, hipStream_t st) {
     if (a.d <= 64) return dispatch_flags<T, 64>(a, st);
+    if (a.d <= 80) return dispatch_flags<T, 96, 5>(a, st);  // five k-steps cover head_dim 80
     if (a.d <= 96) return dispatch_flags<T, 96>(a, st);
     if (a.d <= 128) return dispatch_flags<T, 128>(a, st);
     return SLAPO_ERR_SHAPE;
