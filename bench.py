@@ -50,7 +50,7 @@ FP32_VECTOR_PEAK_TFLOPS = 157.3
 # WRITE_SIZE (KiB per dispatch), each scaled by the same counter's reading for a 256 MiB copy
 # (FETCH_SIZE reads half the copied bytes: factor 2.0; WRITE_SIZE factor 1.0):
 # (43.93e3 * 2.0 + 32.77e3) KiB = 123.5 MB against 101.7 MB algorithmic.  Summary under profiles/.
-DKDV_TRAFFIC_BYTES = (43.93e3 * 2.0 + 32.77e3) * 1024
+DKDV_TRAFFIC_BYTES = (43.46e3 * 2.0 + 32.77e3) * 1024
 HBM_PEAK_GBS = 8000.0      # MI355X HBM3E
 
 WORKLOAD = dict(name="gpt2-medium causal attention fwd+bwd", dtype="fp16", batch=8, seq=1024,
@@ -668,7 +668,7 @@ def main():
                    "heads": cfg["heads"], "head_dim": cfg["head_dim"], "causal": cfg["causal"],
                    "dropout_p": cfg["p"], "flops_per_step": 14 * d * n_pairs},
         "frac_of_mfma_peak": value / MFMA_PEAK_TFLOPS,
-        "roofline": {"bound": "mfma", "kernel": "attn_bwd_kernel<f16,64,0,0,1> (dK/dV)",
+        "roofline": {"bound": "mfma", "kernel": "attn_bwd_kernel<f16,64,0,0,1,4> (dK/dV)",
                      "achieved": achieved,
                      "peak": MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / MFMA_PEAK_TFLOPS, "traffic": DKDV_TRAFFIC_BYTES,
@@ -677,9 +677,9 @@ def main():
                           "raw_event_intervals_ms": seg_raw,
                           "sum_of_kernels_ms": sum(seg_ms)},
     }
-    result["kernels"] = [kern("attn_fwd_kernel<f16,64,0,0,0>", 4 * d * n_pairs, seg_ms[0]),
-                         kern("attn_bwd_kernel<f16,64,0,0,1> (dK/dV)", bwd_flops, seg_ms[2]),
-                         kern("attn_bwd_dq_kernel<f16,64,0,0,true>", 6 * d * n_pairs, seg_ms[1])]
+    result["kernels"] = [kern("attn_fwd_kernel<f16,64,0,0,0,4>", 4 * d * n_pairs, seg_ms[0]),
+                         kern("attn_bwd_kernel<f16,64,0,0,1,4> (dK/dV)", bwd_flops, seg_ms[2]),
+                         kern("attn_bwd_dq_kernel<f16,64,0,0,true,4>", 6 * d * n_pairs, seg_ms[1])]
     with_cpu = not args.no_cpu_baseline
     if not args.no_epilogues:
         result["epilogue"] = bench_epilogues(device)
