@@ -388,8 +388,8 @@ __global__ __launch_bounds__(kThreads, (kStagger && DPAD > 64 ? 1 : 2)) void att
     // Hand-scheduled version of tile_body for tiles without masks: the LDS operands of each group
     // of matrix instructions are requested one phase before the group runs, and scheduling fences
     // keep the compiler from sinking the requests back down to their uses.
-    auto tile_body_fast = [&](const T* kt, const T* vt, int t) __attribute__((always_inline)) {
-        std::integral_constant<int, 0> none;
+    auto tile_body_fast = [&](const T* kt, const T* vt, int t, auto mask_tag)
+                              __attribute__((always_inline)) {
         frag_t kr0[DK], vr0[DK], kr1[DK], vr1[DK], kq0[2 * DV], kq1[2 * DV];
         f32x16_t s0, s1, p0, p1;
         uint32_t dw0[8], dw1[8];
@@ -435,14 +435,14 @@ __global__ __launch_bounds__(kThreads, (kStagger && DPAD > 64 ? 1 : 2)) void att
         __builtin_amdgcn_sched_barrier(0);
         cols(0, kq0);
         mma_rows(kr1, qf, s_init, s1);
-        half_exp(s0, t, 0, none);
+        half_exp(s0, t, 0, mask_tag);
         __builtin_amdgcn_sched_barrier(0);
         cols(1, kq1);
         mma_rows(vr1, gf, dp_init, p1);
         half_ds(s0, p0, t, 0, mw0, dw0);
         __builtin_amdgcn_sched_barrier(0);
         mma_cols(kq0, dw0);
-        half_exp(s1, t, 1, none);
+        half_exp(s1, t, 1, mask_tag);
         half_ds(s1, p1, t, 1, mw1, dw1);
         __builtin_amdgcn_sched_barrier(0);
         mma_cols(kq1, dw1);
@@ -473,16 +473,30 @@ __global__ __launch_bounds__(kThreads, (kStagger && DPAD > 64 ? 1 : 2)) void att
         bias_tile = bias_lds + (r & 1) * kBN;
         if constexpr (kFast) {
             if constexpr (kStagger)
-                tile_body_fast(kt, vt, t);
+                tile_body_fast(kt, vt, t, std::integral_constant<int, 0>{});
             else
                 tile_body(kt, vt, t, std::integral_constant<int, 0>{});
         } else if (tile_active(t)) {
-            if (!tile_needs_mask(t))
-                tile_body(kt, vt, t, std::integral_constant<int, 0>{});
-            else if (a.window > 0)
-                tile_body(kt, vt, t, std::integral_constant<int, 2>{});
-            else
-                tile_body(kt, vt, t, std::integral_constant<int, 1>{});
+            // One wavefront per SIMD (head_dim 128, 412-484 registers): nothing else hides the
+            // latencies of a masked tile, so it runs the hand-scheduled body as well (dQ at bf16 B4
+            // S2048 H16 D128, window 256, p 0.1: 90.8 -> 86.5 us).  With two wavefronts per SIMD
+            // the extra copies of that body cost registers (246 -> 256 and 16 spilled at head_dim
+            // 64) and gain nothing.
+            if constexpr (kStagger && DPAD > 96 && kDrop != 2) {
+                if (!tile_needs_mask(t))
+                    tile_body_fast(kt, vt, t, std::integral_constant<int, 0>{});
+                else if (a.window > 0)
+                    tile_body_fast(kt, vt, t, std::integral_constant<int, 2>{});
+                else
+                    tile_body_fast(kt, vt, t, std::integral_constant<int, 1>{});
+            } else {
+                if (!tile_needs_mask(t))
+                    tile_body(kt, vt, t, std::integral_constant<int, 0>{});
+                else if (a.window > 0)
+                    tile_body(kt, vt, t, std::integral_constant<int, 2>{});
+                else
+                    tile_body(kt, vt, t, std::integral_constant<int, 1>{});
+            }
         }
         if (have_next) {
             ks.fix((t + 1) * kBN, a.sk, a.d);
