@@ -611,3 +611,38 @@ def test_backward_is_bitwise_reproducible_and_stages_compose():
         assert not torch.isnan(a.float()).any()
         assert torch.equal(a, b_)
         assert torch.equal(a, c)
+
+
+# ---- seeded sweep over the whole call surface --------------------------------------------------
+@pytest.mark.parametrize("seed", range(40))
+def test_random_configurations_against_the_oracle(seed):
+    """One random configuration per seed: type, sizes (sequence lengths off the tile sizes,
+    head_dim any multiple of 8 up to 128 -- 72 and 80 run five k-steps of the 96-wide kernels),
+    mask layout, causal flag, local window and dropout; forward and backward against the fp64
+    oracle at the bars of this file."""
+    g = torch.Generator().manual_seed(9000 + seed)
+    r = lambda lo, hi: int(torch.randint(lo, hi + 1, (1,), generator=g))
+    dtype = (torch.float16, torch.bfloat16)[r(0, 1)]
+    b, h = r(1, 2), r(1, 3)
+    d = 8 * r(1, 16)
+    causal = bool(r(0, 1))
+    sq = r(1, 420)
+    sk = sq if causal or r(0, 1) else r(1, 420)
+    layout = ("none", "b11k", "bhqk", "padding")[r(0, 3)]
+    window = 0
+    if causal and layout != "padding" and r(0, 2) == 0:
+        window = r(1, sq + 40)
+    p = (0.0, 0.0, 0.1, 0.25)[r(0, 3)]
+    mk = lambda *shape: torch.randn(*shape, generator=g).to(dtype)
+    q, k, v, do = mk(b, sq, h, d), mk(b, sk, h, d), mk(b, sk, h, d), mk(b, sq, h, d)
+    if layout == "b11k":
+        mask = torch.randn(b, 1, 1, sk, generator=g).to(dtype)
+    elif layout == "bhqk":
+        mask = torch.randn(b, h, sq, sk, generator=g).to(dtype)
+    elif layout == "padding":
+        mask, _ = _padding_mask(b, sk, dtype, g, 1)
+    else:
+        mask = None
+    print(f"seed {seed}: {dtype} b{b} h{h} sq{sq} sk{sk} d{d} causal={causal} window={window} "
+          f"mask={layout} p={p}", flush=True)
+    _check(q, k, v, do, mask, causal, window, dtype, p=p)
