@@ -4,7 +4,7 @@ from .cross_entropy import ParallelCrossEntropy, vocab_parallel_cross_entropy
 from .fused_bias import (BiasGeLUFunction, HipBiasDropoutResidual,
                          HipBiasDropoutResidualLayerNorm, HipBiasGeLU, bias_dropout,
                          bias_dropout_residual, bias_dropout_residual_layer_norm, bias_gelu,
-                         bias_new_gelu)
+                         bias_new_gelu, new_gelu)
 from .linear import (FusedQKV, LinearWithAct, LinearWithDropout, LinearWithSeparateBias,
                      LinearWithSyncFunc)
 from .mlp import FusedMLP

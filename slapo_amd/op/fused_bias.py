@@ -1,7 +1,7 @@
 """Bias epilogues fused with the following activation / dropout, on hand-written HIP kernels.
 
 Same public names and call signatures as the reference's slapo/op/fused_bias.py
-(`BiasGeLUFunction` :13-46, `bias_new_gelu` :63-64, `bias_dropout` :67-74); each runs as ONE
+(`BiasGeLUFunction` :13-46, `new_gelu` :49-60, `bias_new_gelu` :63-64, `bias_dropout` :67-74); each runs as ONE
 streaming kernel per direction instead of a TorchScript / functorch fusion.  Two modules,
 `HipBiasGeLU` and `HipBiasDropoutResidual`, package them with the positional signatures
 (`forward(x, bias)`, `forward(x, bias, residual)`) that `sch.replace(module, subgraph)` needs
@@ -37,6 +37,28 @@ class BiasGeLUFunction(torch.autograd.Function):
 
 def bias_gelu(inp: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
     return BiasGeLUFunction.apply(inp, bias)
+
+
+class _NewGeLU(torch.autograd.Function):
+    """The same kernels with a zero bias and no bias gradient."""
+
+    # pylint: disable=arguments-differ, abstract-method
+    @staticmethod
+    def forward(ctx, inp):
+        zero = inp.new_zeros(inp.shape[-1])
+        ctx.save_for_backward(inp, zero)
+        return K.bias_gelu_fwd(inp, zero)
+
+    @staticmethod
+    def backward(ctx, grad_output):
+        inp, zero = ctx.saved_tensors
+        dx, _ = K.bias_gelu_bwd(grad_output, inp, zero, need_dbias=False)
+        return dx
+
+
+def new_gelu(inp: torch.Tensor) -> torch.Tensor:
+    """HF `gelu_new` (fused_bias.py:49-60) as one kernel per direction."""
+    return _NewGeLU.apply(inp)
 
 
 def bias_new_gelu(inp: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:

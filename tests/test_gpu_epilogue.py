@@ -49,6 +49,21 @@ def test_bias_new_gelu_is_the_same_function():
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_new_gelu_without_a_bias(dtype):
+    """`new_gelu(inp)` of fused_bias.py:49-60 and its autograd-derived gradient."""
+    y, go = _data((3, 50, 136), dtype, n=2)
+    yd = y.cuda().requires_grad_(True)
+    out = op.new_gelu(yd)
+    out.backward(go.cuda())
+    y64 = y.double().requires_grad_(True)
+    ref = OE.new_gelu(y64)
+    ref.backward(go.double())
+    assert out.dtype == dtype and out.shape == y.shape
+    assert_parity(out, ref.detach(), dtype, "new_gelu fwd")
+    assert_parity(yd.grad, y64.grad, dtype, "new_gelu dx")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("shape", [(256, 1024), (4, 33, 1024), (7, 10)])
 @pytest.mark.parametrize("residual", [False, True])
 def test_bias_dropout_residual_p0(dtype, shape, residual):
