@@ -26,7 +26,7 @@
 extern "C" {
 #endif
 
-#define SLAPO_AMD_ABI_VERSION 2
+#define SLAPO_AMD_ABI_VERSION 3
 
 /* status codes */
 #define SLAPO_OK 0
@@ -53,6 +53,16 @@ const char* slapo_amd_status_string(int status);
  * slapo/op/fused_bias.py:74 (bias_dropout) and slapo/op/attention.py:179-180 (xformers_ref).
  * The mask is a pure function of (seed, offset, plan), so it can be regenerated in backward
  * and under activation-checkpoint recompute (slapo/checkpoint.py:79-92).
+ *
+ * (seed, offset) normally travel by value with the call.  A caller whose launches are replayed
+ * (a captured HIP graph) sets plan.rng_state to 16 bytes of device memory holding {seed, offset}
+ * as two uint64 instead: every kernel of the call then reads the pair from there when it runs,
+ * the by-value seed / offset of the call are ignored, and what writes those 16 bytes (ordered
+ * before the call on its stream, e.g. a random-number kernel captured into the same graph)
+ * decides the mask of each replay.  slapo_amd_dropout_plan[_for] leave the field NULL; the host
+ * mirror slapo_amd_dropout_mask_host refuses a plan that has it set (SLAPO_ERR_ARG).  This is
+ * what stands in for the device-side (seed, offset) that ATen's generator hands a captured
+ * launch (the reference's F.dropout calls capture; slapo/op/fused_bias.py:74).
  * ---------------------------------------------------------------------------------------- */
 typedef struct slapo_dropout_plan {
     int64_t numel;            /* elements of the tensor the mask is drawn for                  */
@@ -60,6 +70,7 @@ typedef struct slapo_dropout_plan {
     int32_t vec;              /* elements handled per subsequence per loop trip: 1,2,4,8,16     */
     int32_t calls_per_iter;   /* Philox calls per loop trip = ceil(vec/4) (1 when vec == 1)     */
     int64_t offset_increment; /* amount the generator's offset must be advanced after the draw */
+    const void* rng_state;    /* NULL, or a device address of two uint64 {seed, offset}: see below */
 } slapo_dropout_plan;
 
 /* Host Philox4x32-10 block function (10 rounds).  Pure host code; usable without a GPU. */
@@ -216,7 +227,9 @@ typedef struct slapo_attn_params {
      * through LDS instead of reading it per score: pass a padding mask in that form. */
     int64_t bias_strides[4];
     /* launch plan of the dropout mask over the dense [batch*heads, seqlen_q, seqlen_k] fp32
-     * probability tensor (only read when p_drop > 0) */
+     * probability tensor (only read when p_drop > 0).  With plan.rng_state set the kernels read
+     * {seed, offset} from that device address and ignore the two fields above; a backward call
+     * must then find the values its forward found there. */
     slapo_dropout_plan plan;
     /* Optional (may be NULL), 16-bit types with p_drop > 0 only: device buffer of
      * slapo_amd_attn_keep_mask_bytes(prm) bytes.  The forward call stores the dropout keep bits

@@ -26,10 +26,12 @@ class DropoutPlan(ctypes.Structure):
         ("vec", ctypes.c_int32),
         ("calls_per_iter", ctypes.c_int32),
         ("offset_increment", ctypes.c_int64),
+        ("rng_state", ctypes.c_void_p),
     ]
 
     def as_dict(self):
-        return {name: getattr(self, name) for name, _ in self._fields_}
+        """The launch geometry (everything but the optional device-state pointer)."""
+        return {name: getattr(self, name) for name, _ in self._fields_ if name != "rng_state"}
 
 
 class AttnParams(ctypes.Structure):

@@ -42,7 +42,9 @@ constexpr int kVRing = 2;
 // the K / V tile, and the tile bodies have neither global loads nor branches for them.
 template <typename T, int DPAD, int kBias, int kDrop, bool kStagger, int kSteps>
 __global__ __launch_bounds__(kThreads, (kStagger && DPAD > 64 ? 1 : 2)) void attn_bwd_dq_kernel(
-    const AttnArgs a) {
+    const AttnArgs a_in) {
+    AttnArgs a = a_in;
+    if constexpr (kDrop == 1 || kDrop == 2) resolve_device_state(a.rng);
     typedef typename Mma<T>::frag frag_t;
     typedef TileStage<T, DPAD, kBN, kThreads> Stage;
     constexpr int kPitch = Stage::kPitch;

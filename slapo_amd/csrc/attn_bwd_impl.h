@@ -58,7 +58,9 @@ template <typename T, int DPAD, int kBias, int kDrop, int KB, int kSteps>
 // Two workgroups per CU up to DPAD 96, one at 128 (192 resident accumulator / fragment registers)
 // and at 96 with the forward's keep bits (measured 23-35 % slower with two than with one).
 __global__ __launch_bounds__(kBwdThreads, (bwd_two_per_cu(DPAD, kDrop, KB) ? 2 : 1)) void attn_bwd_kernel(
-    const AttnArgs a) {
+    const AttnArgs a_in) {
+    AttnArgs a = a_in;
+    if constexpr (kDrop == 1 || kDrop == 2) resolve_device_state(a.rng);
     static_assert(kDrop != 3 || KB == 1, "the keep-bit tile holds one word per wavefront and query");
     typedef typename Mma<T>::frag frag_t;
     typedef BwdSmem<T, DPAD> SM;

@@ -79,7 +79,9 @@ __global__ __launch_bounds__(256) void attn_delta_scalar_kernel(const AttnArgs a
 // seqlen_k / 32: every thread then has a word to draw); without one it is the word itself.
 // kExact: any launch geometry of the dropout plan and any seqlen_k (one Philox block per bit).
 template <bool kExact>
-__global__ __launch_bounds__(256) void keep_mask_kernel(const AttnArgs a) {
+__global__ __launch_bounds__(256) void keep_mask_kernel(const AttnArgs a_in) {
+    AttnArgs a = a_in;
+    resolve_device_state(a.rng);
     const int i = blockIdx.x * 256 + threadIdx.x;
     const int bh = blockIdx.z;
     if (i >= a.sq) return;

@@ -37,7 +37,9 @@ __device__ __forceinline__ void load_rows(float (*dst)[DMAX], const float* base,
 }
 
 template <int DMAX>
-__global__ __launch_bounds__(kRows) void attn_f32_fwd_kernel(const AttnArgs a) {
+__global__ __launch_bounds__(kRows) void attn_f32_fwd_kernel(const AttnArgs a_in) {
+    AttnArgs a = a_in;
+    if (a.dropout) resolve_device_state(a.rng);
     __shared__ float ks[kTile][DMAX];
     __shared__ float vs[kTile][DMAX];
     const int bh = blockIdx.y, b = bh / a.heads, h = bh % a.heads;
@@ -101,7 +103,9 @@ __global__ __launch_bounds__(kRows) void attn_f32_fwd_kernel(const AttnArgs a) {
 
 // dQ: thread = query.  dq_i = scale * sum_j ds_ij k_j,  ds = p (dp - delta),  dp = dO_i . v_j
 template <int DMAX>
-__global__ __launch_bounds__(kRows) void attn_f32_dq_kernel(const AttnArgs a) {
+__global__ __launch_bounds__(kRows) void attn_f32_dq_kernel(const AttnArgs a_in) {
+    AttnArgs a = a_in;
+    if (a.dropout) resolve_device_state(a.rng);
     __shared__ float ks[kTile][DMAX];
     __shared__ float vs[kTile][DMAX];
     const int bh = blockIdx.y, b = bh / a.heads, h = bh % a.heads;
@@ -162,7 +166,9 @@ __global__ __launch_bounds__(kRows) void attn_f32_dq_kernel(const AttnArgs a) {
 // dK (kWhich == 0) or dV (kWhich == 1): thread = key, queries stream through LDS.
 //   dv_j = sum_i pdrop_ij dO_i          dk_j = scale * sum_i ds_ij q_i
 template <int DMAX, int kWhich>
-__global__ __launch_bounds__(kRows) void attn_f32_dkv_kernel(const AttnArgs a) {
+__global__ __launch_bounds__(kRows) void attn_f32_dkv_kernel(const AttnArgs a_in) {
+    AttnArgs a = a_in;
+    if (a.dropout) resolve_device_state(a.rng);
     __shared__ float qs[kTile][DMAX];
     __shared__ float gs[kTile][DMAX];
     __shared__ float lse_s[kTile], inv_n_s[kTile];

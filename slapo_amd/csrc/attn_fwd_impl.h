@@ -47,6 +47,7 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
     // 116 -> 96-109 us at bf16 B4 S2048 H16 causal); folding "window" in leaves one masked body.
     AttnArgs a = a_in;
     if constexpr (kWin == 0) a.window = 0;
+    if constexpr (kDrop == 1 || kDrop == 2) resolve_device_state(a.rng);
     typedef typename Mma<T>::frag frag_t;
     typedef TileStage<T, DPAD, kBN, kThreads> Stage;
     constexpr int kPitch = Stage::kPitch;

@@ -120,6 +120,7 @@ inline DropoutState make_dropout_state(const slapo_dropout_plan& plan, double p,
     }
     s.g_shift = s.vec >= 4 ? (s.vec == 4 ? 0 : s.vec == 8 ? 1 : 2) : -1;
     s.inv_keep = p < 1.0 ? (float)(1.0 / (double)(float)(1.0 - p)) : 0.f;
+    s.device_state = static_cast<const uint64_t*>(plan.rng_state);
     return s;
 }
 

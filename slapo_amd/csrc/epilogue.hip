@@ -145,6 +145,7 @@ __global__ __launch_bounds__(256) void bias_dropout_residual_fwd_kernel(
     const T* __restrict__ x, const T* __restrict__ bias, const T* __restrict__ residual,
     T* __restrict__ out, uint64_t n_chunks, uint32_t chunks_per_row, uint32_t row_mask,
     DropoutState s) {
+    if constexpr (kDrop != 0) resolve_device_state(s);
     const uint64_t base = (uint64_t)blockIdx.x * (256 * kDU) + threadIdx.x;
     Chunk<T, V> in[kDU];
     Chunk<T, V> res[kDU];
@@ -295,6 +296,7 @@ __global__ __launch_bounds__(256) void bias_dropout_bwd_kernel(const T* __restri
                                                                int want_sum, int write_dx,
                                                                int rows_per_block,
                                                                DropoutState s) {
+    if constexpr (kDrop != 0) resolve_device_state(s);
     colsum_walk<T, V>(rows, cols, partial, want_sum != 0, rows_per_block,
                       [&](int64_t r, int64_t col0, float* acc) {
                           const int64_t off = r * cols + col0;
@@ -404,6 +406,7 @@ __global__ __launch_bounds__(256) void bias_dropout_residual_ln_fwd_kernel(
     const T* __restrict__ gamma, const T* __restrict__ beta, T* __restrict__ z_out,
     T* __restrict__ y, float* __restrict__ mean_out, float* __restrict__ rstd_out, int64_t rows,
     int cols, float eps, DropoutState s) {
+    if constexpr (kDrop != 0) resolve_device_state(s);
     constexpr int kRows = 256 / TPR;  // rows per block
     __shared__ float red[2][4];
     const int sub = threadIdx.x % TPR;
@@ -509,6 +512,7 @@ void bias_dropout_residual_ln_bwd_kernel(
     const T* __restrict__ dy, const T* __restrict__ z, const float* __restrict__ mean,
     const float* __restrict__ rstd, const T* __restrict__ gamma, T* __restrict__ dx,
     T* __restrict__ dres, float* __restrict__ partial, int64_t rows, int cols, DropoutState s) {
+    if constexpr (kDrop != 0) resolve_device_state(s);
     static_assert(TPR == 256 ? kThreads == 256 : (kThreads == 256 || kThreads == 512),
                   "a block is one wide row, or four or eight wavefront rows");
     constexpr int kRows = kThreads / TPR;  // rows in flight per block

@@ -61,7 +61,23 @@ struct DropoutState {
     int32_t t_shift;          // log2(T) when T is a power of two, else -1
     int32_t g_shift;          // log2(vec / 4) when vec >= 4, else -1
     float inv_keep;           // 1 / (1 - p)
+    // NULL, or device memory holding {seed, offset}: a kernel then takes key and base counter
+    // from there (resolve_device_state) instead of the three fields above
+    const uint64_t* device_state;
 };
+
+#if defined(__HIPCC__)
+// First statement of every kernel that draws: a uniform branch and one 16-byte uniform read.
+__device__ __forceinline__ void resolve_device_state(DropoutState& s) {
+    if (s.device_state != nullptr) {
+        const uint64_t seed = s.device_state[0];
+        const uint64_t offset = s.device_state[1];
+        s.key0 = (uint32_t)seed;
+        s.key1 = (uint32_t)(seed >> 32);
+        s.base_counter = offset >> 2;
+    }
+}
+#endif
 
 SLAPO_HD void split_by_threads(const DropoutState& s, uint64_t v, uint64_t& thread,
                                uint64_t& trip) {

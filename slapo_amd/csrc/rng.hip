@@ -45,6 +45,7 @@ extern "C" int slapo_amd_dropout_plan_for(int64_t numel, int elem_bytes, int64_t
     plan->calls_per_iter = vec == 1 ? 1 : (vec + 3) / 4;
     const int64_t unroll = 4;
     plan->offset_increment = ((numel - 1) / (block * grid * unroll) + 1) * unroll;
+    plan->rng_state = nullptr;
     return SLAPO_OK;
 }
 
@@ -91,6 +92,7 @@ extern "C" int slapo_amd_dropout_mask_host(uint8_t* mask, const slapo_dropout_pl
                                            double p, uint64_t seed, uint64_t offset) {
     if (!mask || !plan || !plan_ok(plan, plan->numel)) return SLAPO_ERR_ARG;
     if (!(p >= 0.0 && p <= 1.0)) return SLAPO_ERR_ARG;
+    if (plan->rng_state != nullptr) return SLAPO_ERR_ARG;  // device memory: not readable here
     const DropoutState s = make_dropout_state(*plan, p, seed, offset);
     const int64_t n = plan->numel;
     if (s.vec >= 4 && n % 4 == 0) {
@@ -106,6 +108,7 @@ extern "C" int slapo_amd_dropout_mask_host(uint8_t* mask, const slapo_dropout_pl
 
 __global__ __launch_bounds__(256) void dropout_mask_kernel(uint8_t* __restrict__ mask,
                                                            int64_t numel, DropoutState s) {
+    resolve_device_state(s);
     const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (s.vec >= 4) {
         const int64_t g = tid;

@@ -73,6 +73,22 @@ def dropout_plan(numel: int, elem_bytes: int, device) -> DropoutPlan:
     return _plan_cached(int(numel), int(elem_bytes), int(idx))
 
 
+def _plan_ref(plan, rng_state=None):
+    """The plan as a call argument.  `rng_state` (a device tensor of two 64-bit integers, {seed,
+    offset}) makes the kernels read the pair from device memory when they run -- what a captured
+    graph needs -- instead of taking the call's seed / offset values."""
+    if plan is None:
+        return None
+    if rng_state is None:
+        return ctypes.byref(plan)
+    if (rng_state.dtype not in (torch.int64, torch.uint64) or rng_state.numel() != 2
+            or not rng_state.is_cuda or not rng_state.is_contiguous()):
+        raise ValueError("rng_state must be a contiguous device tensor of two 64-bit integers")
+    own = DropoutPlan.from_buffer_copy(plan)
+    own.rng_state = rng_state.data_ptr()
+    return ctypes.byref(own)
+
+
 def _rows_cols(x, bias):
     cols = x.shape[-1]
     if bias.ndim != 1 or bias.shape[0] != cols:
@@ -122,7 +138,7 @@ def bias_gelu_bwd(grad, y, bias, need_dbias=True):
     return dx, dbias
 
 
-def bias_dropout_residual_fwd(x, bias, residual, p, seed, offset, plan):
+def bias_dropout_residual_fwd(x, bias, residual, p, seed, offset, plan, rng_state=None):
     _require_device(x, bias, residual)
     x = x.contiguous()
     bias, residual = _same_dtype(x, bias.contiguous(),
@@ -137,13 +153,13 @@ def bias_dropout_residual_fwd(x, bias, residual, p, seed, offset, plan):
         rc = _lib.load().slapo_amd_bias_dropout_residual_fwd(
             _ptr(x), _ptr(bias), _ptr(residual), _ptr(out), rows, cols,
             _lib.dtype_code(x.dtype), float(p), seed, offset,
-            ctypes.byref(plan) if plan is not None else None, _stream())
+            _plan_ref(plan, rng_state), _stream())
     _lib.check(rc, "slapo_amd_bias_dropout_residual_fwd")
     return out
 
 
 def bias_dropout_residual_bwd(grad, bias_like, p, seed, offset, plan, need_dx=True,
-                              need_dbias=True):
+                              need_dbias=True, rng_state=None):
     _require_device(grad)
     grad = grad.contiguous()
     cols = grad.shape[-1]
@@ -157,7 +173,7 @@ def bias_dropout_residual_bwd(grad, bias_like, p, seed, offset, plan, need_dx=Tr
         rc = _lib.load().slapo_amd_bias_dropout_residual_bwd(
             _ptr(grad), _ptr(dx), _ptr(dbias), _ptr(ws), nbytes, rows, cols,
             _lib.dtype_code(grad.dtype), float(p), seed, offset,
-            ctypes.byref(plan) if plan is not None else None, _stream())
+            _plan_ref(plan, rng_state), _stream())
     _lib.check(rc, "slapo_amd_bias_dropout_residual_bwd")
     if dbias is not None and dbias.dtype != bias_like.dtype:
         dbias = dbias.to(bias_like.dtype)
@@ -165,7 +181,7 @@ def bias_dropout_residual_bwd(grad, bias_like, p, seed, offset, plan, need_dx=Tr
 
 
 def bias_dropout_residual_ln_fwd(x, bias, residual, weight, ln_bias, eps, p, seed, offset, plan,
-                                 save_for_backward=True):
+                                 save_for_backward=True, rng_state=None):
     """Returns (y, z, mean, rstd); the last three are None without save_for_backward."""
     _require_device(x, bias, residual, weight, ln_bias)
     x = x.contiguous()
@@ -192,14 +208,14 @@ def bias_dropout_residual_ln_fwd(x, bias, residual, weight, ln_bias, eps, p, see
         rc = _lib.load().slapo_amd_bias_dropout_residual_ln_fwd(
             _ptr(x), _ptr(bias), _ptr(residual), _ptr(weight), _ptr(ln_bias), _ptr(z), _ptr(y),
             _ptr(mean), _ptr(rstd), rows, cols, _lib.dtype_code(x.dtype), float(eps), float(p),
-            seed, offset, ctypes.byref(plan) if plan is not None else None, _stream())
+            seed, offset, _plan_ref(plan, rng_state), _stream())
     _lib.check(rc, "slapo_amd_bias_dropout_residual_ln_fwd")
     return y, z, mean, rstd
 
 
 def bias_dropout_residual_ln_bwd(grad, z, mean, rstd, weight, p, seed, offset, plan, need_dx=True,
                                  need_dres=True, need_dweight=True, need_dln_bias=True,
-                                 need_dbias=True):
+                                 need_dbias=True, rng_state=None):
     """Returns (dx, dresidual, dweight, dln_bias, dbias); entries not asked for are None."""
     _require_device(grad, z, mean, rstd, weight)
     grad = grad.contiguous()
@@ -226,7 +242,7 @@ def bias_dropout_residual_ln_bwd(grad, z, mean, rstd, weight, p, seed, offset, p
             _ptr(grad), _ptr(z), _ptr(mean), _ptr(rstd), _ptr(weight), _ptr(dx), _ptr(dres),
             _ptr(dw), _ptr(dlb), _ptr(db), _ptr(ws), nbytes, rows, cols,
             _lib.dtype_code(z.dtype), float(p), seed, offset,
-            ctypes.byref(plan) if plan is not None else None, _stream())
+            _plan_ref(plan, rng_state), _stream())
     _lib.check(rc, "slapo_amd_bias_dropout_residual_ln_bwd")
     return outs
 
@@ -269,13 +285,13 @@ def vocab_ce_bwd(logits, target, row_max, inv_sum_exp, grad_loss, vocab_start=0,
     return grad
 
 
-def dropout_mask(numel, elem_bytes, p, seed, offset, device):
+def dropout_mask(numel, elem_bytes, p, seed, offset, device, rng_state=None):
     """Boolean keep-mask [numel] drawn on the device (debugging / test aid)."""
     plan = dropout_plan(numel, elem_bytes, device)
     mask = torch.empty(numel, dtype=torch.uint8, device=device)
     with _on(device):
-        rc = _lib.load().slapo_amd_dropout_mask(_ptr(mask), ctypes.byref(plan), float(p), seed,
-                                                offset, _stream())
+        rc = _lib.load().slapo_amd_dropout_mask(_ptr(mask), _plan_ref(plan, rng_state), float(p),
+                                                seed, offset, _stream())
     _lib.check(rc, "slapo_amd_dropout_mask")
     return mask.bool()
 
@@ -311,7 +327,7 @@ _PARAMS_CACHE = {}
 
 
 def make_attn_params(q, k, v, o, bias, causal, window, scale, p, seed, offset, plan,
-                     keep_mask=None):
+                     keep_mask=None, rng_state=None):
     """The parameter struct of one attention call.  Everything but (seed, offset, keep_mask) is a
     function of the problem geometry and is cached."""
     key = (q.dtype, q.shape, k.shape[1], q.stride(), k.stride(), v.stride(), o.stride(),
@@ -344,6 +360,11 @@ def make_attn_params(q, k, v, o, bias, causal, window, scale, p, seed, offset, p
     prm.offset = int(offset)
     if keep_mask is not None:
         prm.keep_mask = keep_mask.data_ptr()
+    if rng_state is not None:
+        if (rng_state.dtype not in (torch.int64, torch.uint64) or rng_state.numel() != 2
+                or not rng_state.is_cuda or not rng_state.is_contiguous()):
+            raise ValueError("rng_state must be a contiguous device tensor of two 64-bit integers")
+        prm.plan.rng_state = rng_state.data_ptr()
     return prm
 
 
@@ -358,7 +379,8 @@ def prepare_bias(attention_mask, b, h, sq, sk):
     return m.expand(b, h, sq, sk)
 
 
-def attn_fwd(q, k, v, bias, causal, window, scale, p, seed, offset, plan, save_mask=None):
+def attn_fwd(q, k, v, bias, causal, window, scale, p, seed, offset, plan, save_mask=None,
+             rng_state=None):
     """Returns (o, lse, (q, k, v) as consumed); when save_mask is given (True / False) a fourth
     item: the dropout keep bits for attn_bwd, or None (save_mask False, p == 0, fp32)."""
     _require_device(q, k, v, bias)
@@ -366,7 +388,8 @@ def attn_fwd(q, k, v, bias, causal, window, scale, p, seed, offset, plan, save_m
     b, sq, h, d = q.shape
     o = torch.empty((b, sq, h, d), dtype=q.dtype, device=q.device)
     lse = torch.empty((b, h, sq), dtype=torch.float32, device=q.device)
-    prm = make_attn_params(q, k, v, o, bias, causal, window, scale, p, seed, offset, plan)
+    prm = make_attn_params(q, k, v, o, bias, causal, window, scale, p, seed, offset, plan,
+                           rng_state=rng_state)
     keep_mask = None
     if save_mask and o.numel():
         nbytes = _lib.load().slapo_amd_attn_keep_mask_bytes(ctypes.byref(prm))
@@ -384,7 +407,7 @@ def attn_fwd(q, k, v, bias, causal, window, scale, p, seed, offset, plan, save_m
 
 
 def attn_bwd(dout, q, k, v, bias, o, lse, causal, window, scale, p, seed, offset, plan,
-             keep_mask=None):
+             keep_mask=None, rng_state=None):
     _require_device(dout, q, k, v, o, lse, bias)
     dout = dout if dout.stride() == o.stride() else dout.contiguous()
     if dout.stride() != o.stride():
@@ -393,7 +416,7 @@ def attn_bwd(dout, q, k, v, bias, o, lse, causal, window, scale, p, seed, offset
     dk = torch.empty(k.shape, dtype=k.dtype, device=k.device)
     dv = torch.empty(v.shape, dtype=v.dtype, device=v.device)
     prm = make_attn_params(q, k, v, o, bias, causal, window, scale, p, seed, offset, plan,
-                           keep_mask)
+                           keep_mask, rng_state)
     if dq.numel() and dk.numel():
         lib = _lib.load()
         nbytes = lib.slapo_amd_attn_bwd_workspace_bytes(ctypes.byref(prm))

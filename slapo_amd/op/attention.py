@@ -28,7 +28,7 @@ import torch
 import torch.nn.functional as F
 from torch import nn
 
-from ..random import draw_philox
+from ..random import draw_philox, draw_philox_state
 from . import _kernels as K
 from .fused_bias import bias_dropout
 
@@ -66,29 +66,30 @@ class _HipAttention(torch.autograd.Function):
     def forward(ctx, q, k, v, bias, causal, window, scale, p):
         b, sq, h, _ = q.shape
         sk = k.shape[1]
-        plan, seed, offset = None, 0, 0
+        plan, seed, offset, rng_state = None, 0, 0, None
         if b * h * sq * sk == 0:
             p = 0.0  # nothing to drop, and F.dropout leaves the generator alone for an empty tensor
         if p > 0.0:
             plan = K.dropout_plan(b * h * sq * sk, 4, q.device)
             if p < 1.0:
-                seed, offset = draw_philox(plan.offset_increment, q.device)
+                seed, offset, rng_state = draw_philox_state(plan.offset_increment, q.device)
         save_mask = SAVE_DROPOUT_MASK and 0.0 < p < 1.0 and any(ctx.needs_input_grad[:3])
         if save_mask:
             mask_bytes = b * h * ((sk + 31) // 32) * ((sq + 3) // 4 * 4) * 4
             save_mask = mask_bytes <= SAVE_DROPOUT_MASK_MAX_BYTES
         out, lse, (q, k, v), keep_mask = K.attn_fwd(q, k, v, bias, causal, window, scale, p, seed,
-                                                    offset, plan, save_mask=save_mask)
-        ctx.save_for_backward(q, k, v, bias, out, lse, keep_mask)
+                                                    offset, plan, save_mask=save_mask,
+                                                    rng_state=rng_state)
+        ctx.save_for_backward(q, k, v, bias, out, lse, keep_mask, rng_state)
         ctx.cfg = (causal, window, scale, p, seed, offset, plan)
         return out
 
     @staticmethod
     def backward(ctx, dout):
-        q, k, v, bias, out, lse, keep_mask = ctx.saved_tensors
+        q, k, v, bias, out, lse, keep_mask, rng_state = ctx.saved_tensors
         causal, window, scale, p, seed, offset, plan = ctx.cfg
         dq, dk, dv = K.attn_bwd(dout, q, k, v, bias, out, lse, causal, window, scale, p, seed,
-                                offset, plan, keep_mask)
+                                offset, plan, keep_mask, rng_state)
         return dq, dk, dv, None, None, None, None, None
 
 

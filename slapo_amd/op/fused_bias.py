@@ -12,7 +12,7 @@ from __future__ import annotations
 import torch
 from torch import nn
 
-from ..random import draw_philox
+from ..random import draw_philox_state
 from . import _kernels as K
 
 
@@ -71,18 +71,20 @@ class _BiasDropoutResidual(torch.autograd.Function):
     # pylint: disable=arguments-differ, abstract-method
     @staticmethod
     def forward(ctx, x, bias, residual, p):
-        plan, seed, offset = None, 0, 0
+        plan, seed, offset, rng_state = None, 0, 0, None
         if x.numel() == 0:
             p = 0.0  # nothing to drop, and F.dropout leaves the generator alone for an empty tensor
         if 0.0 < p:
             plan = K.dropout_plan(x.numel(), x.element_size(), x.device)
             if p < 1.0:
                 # The generator moves exactly as it would for F.dropout on this tensor.
-                seed, offset = draw_philox(plan.offset_increment, x.device)
+                seed, offset, rng_state = draw_philox_state(plan.offset_increment, x.device)
         ctx.p, ctx.seed, ctx.offset, ctx.plan = p, seed, offset, plan
+        ctx.rng_state = rng_state  # a non-differentiable two-element tensor, or None
         ctx.bias_like = bias
         ctx.has_residual = residual is not None
-        return K.bias_dropout_residual_fwd(x, bias, residual, p, seed, offset, plan)
+        return K.bias_dropout_residual_fwd(x, bias, residual, p, seed, offset, plan,
+                                           rng_state=rng_state)
 
     @staticmethod
     def backward(ctx, grad_output):
@@ -94,7 +96,7 @@ class _BiasDropoutResidual(torch.autograd.Function):
             else:
                 dx, dbias = K.bias_dropout_residual_bwd(
                     grad_output, ctx.bias_like, ctx.p, ctx.seed, ctx.offset, ctx.plan,
-                    need_dx=need_dx, need_dbias=need_dbias)
+                    need_dx=need_dx, need_dbias=need_dbias, rng_state=ctx.rng_state)
         dres = grad_output if (ctx.has_residual and ctx.needs_input_grad[2]) else None
         return dx, dbias, dres, None
 
@@ -119,18 +121,19 @@ class _BiasDropoutResidualLayerNorm(torch.autograd.Function):
     # pylint: disable=arguments-differ, abstract-method
     @staticmethod
     def forward(ctx, x, bias, residual, weight, ln_bias, p, eps):
-        plan, seed, offset = None, 0, 0
+        plan, seed, offset, rng_state = None, 0, 0, None
         if x.numel() == 0:
             p = 0.0  # nothing to drop, and F.dropout leaves the generator alone for an empty tensor
         if 0.0 < p:
             plan = K.dropout_plan(x.numel(), x.element_size(), x.device)
             if p < 1.0:
                 # The generator moves exactly as it would for F.dropout on this tensor.
-                seed, offset = draw_philox(plan.offset_increment, x.device)
+                seed, offset, rng_state = draw_philox_state(plan.offset_increment, x.device)
         need_grad = any(ctx.needs_input_grad[:5])
         y, z, mean, rstd = K.bias_dropout_residual_ln_fwd(
             x, bias, residual, weight, ln_bias, eps, p, seed, offset, plan,
-            save_for_backward=need_grad)
+            save_for_backward=need_grad, rng_state=rng_state)
+        ctx.rng_state = rng_state  # a non-differentiable two-element tensor, or None
         ctx.cfg = (p, seed, offset, plan, bias is not None, residual is not None)
         ctx.dtypes = tuple(t.dtype if t is not None else None for t in (bias, weight, ln_bias))
         ctx.save_for_backward(z, mean, rstd, weight)
@@ -144,7 +147,7 @@ class _BiasDropoutResidualLayerNorm(torch.autograd.Function):
         dx, dres, dw, dlb, db = K.bias_dropout_residual_ln_bwd(
             grad_output, z, mean, rstd, weight, p, seed, offset, plan, need_dx=need[0],
             need_dres=has_residual and need[2], need_dweight=need[3], need_dln_bias=need[4],
-            need_dbias=has_bias and need[1])
+            need_dbias=has_bias and need[1], rng_state=ctx.rng_state)
         cast = lambda t, dt: t if t is None or t.dtype == dt else t.to(dt)
         return (dx, cast(db, ctx.dtypes[0]), dres, cast(dw, ctx.dtypes[1]),
                 cast(dlb, ctx.dtypes[2]), None, None)

@@ -140,14 +140,35 @@ def draw_philox(offset_increment: int, device=None):
         raise ValueError("Philox offset increments are multiples of 4")
     if torch.cuda.is_available() and torch.cuda.is_current_stream_capturing():
         # The pair is read on the host and baked into the launch: a captured graph would replay
-        # one and the same mask.  Capture the C-ABI entry points with dropout off, or with
-        # caller-supplied (seed, offset) pairs, instead.
+        # one and the same mask.  `draw_philox_state` is the capturable form.
         raise RuntimeError(
-            "slapo_amd: dropout with p > 0 draws (seed, offset) from the device generator on the "
-            "host and cannot be captured into a graph"
+            "slapo_amd: draw_philox reads (seed, offset) from the device generator on the host "
+            "and cannot be captured into a graph; use draw_philox_state"
         )
     gen = DeviceGeneratorBackend._gen(device)
     seed = gen.initial_seed()
     offset = gen.get_offset()
     gen.set_offset(offset + offset_increment)
     return seed, offset
+
+
+def draw_philox_state(offset_increment: int, device=None):
+    """`draw_philox` for the ops of this package: (seed, offset, state).
+
+    Outside a graph capture `state` is None and (seed, offset) are `draw_philox`'s.  While the
+    current stream is being captured the pair cannot travel by value (every replay would draw one
+    and the same mask), so it lives in device memory instead: `state` is a tensor of two 64-bit
+    integers written by a torch random kernel that is captured with the launch and draws from the
+    device's default generator, which torch re-seeds for every replay of the graph.  The kernels
+    of the op (forward and backward) read {seed, offset} from it when they run; the by-value
+    seed and offset are 0 and unused.  A replay's mask is then a function of the generator's
+    state at that replay -- fresh per replay, repeatable after `torch.cuda.manual_seed` -- though
+    not the mask an eager call would draw from the same state."""
+    if torch.cuda.is_available() and torch.cuda.is_current_stream_capturing():
+        if offset_increment % 4 != 0:
+            raise ValueError("Philox offset increments are multiples of 4")
+        dev = torch.device("cuda", torch.cuda.current_device()) if device is None else device
+        state = torch.randint(0, 2 ** 62, (2,), dtype=torch.int64, device=dev)
+        return 0, 0, state
+    seed, offset = draw_philox(offset_increment, device)
+    return seed, offset, None

@@ -34,7 +34,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_abi_version_and_status_strings():
     lib = _lib.load()
-    assert lib.slapo_amd_abi_version() == 2
+    assert lib.slapo_amd_abi_version() == 3
     assert lib.slapo_amd_status_string(0) == b"ok"
     for code in range(-7, 0):
         assert lib.slapo_amd_status_string(code) not in (b"ok", b"unknown status")
@@ -42,8 +42,8 @@ def test_abi_version_and_status_strings():
 
 def test_struct_layout_matches_header():
     # sizes the C compiler produces for the two PODs (natural alignment, no packing)
-    assert ctypes.sizeof(DropoutPlan) == 32
-    assert ctypes.sizeof(_lib.AttnParams) == 4 * 8 + 2 * 4 + 2 * 8 + 16 * 8 + 32 + 8
+    assert ctypes.sizeof(DropoutPlan) == 40
+    assert ctypes.sizeof(_lib.AttnParams) == 4 * 8 + 2 * 4 + 2 * 8 + 16 * 8 + 40 + 8
 
 
 def test_host_philox_known_answers():
@@ -153,3 +153,17 @@ def test_compute_entry_points_validate_before_touching_the_device():
     assert lib.slapo_amd_attn_keep_mask_bytes(ctypes.byref(prm)) == 2 * 3 * 3 * 72 * 4
     prm.dtype = 0
     assert lib.slapo_amd_attn_keep_mask_bytes(ctypes.byref(prm)) == 0
+
+
+def test_host_mask_mirror_refuses_a_device_resident_pair():
+    """plan.rng_state names device memory; the host mirror cannot read it and says so."""
+    lib = _lib.load()
+    plan = DropoutPlan()
+    assert lib.slapo_amd_dropout_plan_for(64, 2, 256, 256, 2048, ctypes.byref(plan)) == 0
+    assert plan.rng_state is None
+    host = np.zeros(64, dtype=np.uint8)
+    assert lib.slapo_amd_dropout_mask_host(host.ctypes.data_as(ctypes.c_void_p),
+                                           ctypes.byref(plan), 0.5, 1, 0) == 0
+    plan.rng_state = 0x1000
+    assert lib.slapo_amd_dropout_mask_host(host.ctypes.data_as(ctypes.c_void_p),
+                                           ctypes.byref(plan), 0.5, 1, 0) == -4
