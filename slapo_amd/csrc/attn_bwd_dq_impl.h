@@ -180,7 +180,11 @@ __global__ __launch_bounds__(kThreads, (kStagger && DPAD > 64 ? 1 : 2)) void att
         dp_init[r] = kAccInit && kDrop == 0 ? -delta : 0.f;
     }
     const float lse_sub = kAccInit ? 0.f : lse2;
-    const float delta_sub = kAccInit && kDrop == 0 ? 0.f : delta;
+    // With dropout dS = P (M dP / (1 - p) - delta) is taken as (P (M dP - delta (1 - p))) / (1 - p):
+    // the kept dP stay as they are (dropped ones become +0, two instructions each), delta is
+    // scaled once per row and the factor goes onto the dQ rows when they are written.
+    const float keep_prob = a.rng.inv_keep > 0.f ? 1.0f / a.rng.inv_keep : 0.f;
+    const float delta_sub = kAccInit && kDrop == 0 ? 0.f : (kDrop != 0 ? delta * keep_prob : delta);
 
     f32x16_t dq_acc[DV];
 #pragma unroll
@@ -347,8 +351,7 @@ __global__ __launch_bounds__(kThreads, (kStagger && DPAD > 64 ? 1 : 2)) void att
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
             float d = dp[r];
-            if constexpr (kDrop != 0)
-                d = ((word_g >> acc_row(r, 0)) & 1u) ? d * a.rng.inv_keep : 0.f;
+            if constexpr (kDrop != 0) d = keep_or_zero(d, word_g, acc_row(r, 0));
             if constexpr (kAccInit && kDrop == 0)
                 dv[r] = p[r] * d;  // delta already subtracted by the matrix pipe
             else
@@ -525,7 +528,8 @@ __global__ __launch_bounds__(kThreads, (kStagger && DPAD > 64 ? 1 : 2)) void att
     if (wq0 < a.sq) {
         T* dq_row0 =
             reinterpret_cast<T*>(a.dq) + b * a.dqs[0] + (int64_t)wq0 * a.dqs[1] + h * a.dqs[2];
-        store_block_via_lds<T, DPAD, kPitch>(dq_acc, a.scale * inv_n, k_lds + wave * 32 * kPitch,
+        const float out_scale = (kDrop != 0 ? a.scale * a.rng.inv_keep : a.scale) * inv_n;
+        store_block_via_lds<T, DPAD, kPitch>(dq_acc, out_scale, k_lds + wave * 32 * kPitch,
                                              dq_row0, a.dqs[1], a.sq - wq0, a.d);
     }
 }

@@ -102,6 +102,9 @@ __global__ __launch_bounds__(kBwdThreads, (bwd_two_per_cu(DPAD, kDrop, KB) ? 2 :
     const T* g_base = reinterpret_cast<const T*>(a.dout) + b * a.os[0] + h * a.os[2];
     const float* lse_base = a.lse + (int64_t)bh * a.sq;
     const float* delta_base = a.delta + (int64_t)bh * a.sq;
+    // With dropout dS = P (M dP / (1 - p) - delta) is taken as (P (M dP - delta (1 - p))) / (1 - p):
+    // delta is scaled when it is staged and the factor goes onto the dK rows when they are written.
+    const float keep_prob = a.rng.inv_keep > 0.f ? 1.0f / a.rng.inv_keep : 0.f;
 
     // ---- resident fragments ----
     // Loaded with clamped addresses and masked once the first query tile has been requested too,
@@ -217,7 +220,7 @@ __global__ __launch_bounds__(kBwdThreads, (bwd_two_per_cu(DPAD, kDrop, KB) ? 2 :
             const float v = (threadIdx.x < kBwdBM)
                                 ? (ok ? -(kBias ? lse_reference(r.stat, kLog2e) : r.stat * kLog2e)
                                       : -INFINITY)
-                                : (ok ? (kDrop == 0 ? -r.stat : r.stat) : 0.f);
+                                : (ok ? (kDrop == 0 ? -r.stat : r.stat * keep_prob) : 0.f);
             stat_lds[buf * 2 * kBwdBM + (threadIdx.x & kBwdBM) + row_slot(threadIdx.x & (kBwdBM - 1))] = v;
         }
         if constexpr (kDrop == 3)
@@ -437,12 +440,12 @@ __global__ __launch_bounds__(kBwdThreads, (bwd_two_per_cu(DPAD, kDrop, KB) ? 2 :
                     float d = dp[kb][4 * r4 + e];
                     float pd = pe;
                     if constexpr (kDrop != 0) {
-                        // dropped pairs become +0; dV takes its factor 1 / (1 - p) when it is
-                        // written, dP takes it here
+                        // dropped pairs become +0; dV and dK take the factor 1 / (1 - p) when
+                        // they are written (the staged delta carries 1 - p instead)
                         const uint32_t bits = kDrop == 3 ? w4[e] : wq[kb][e];
                         const uint32_t pos = kDrop == 3 ? (uint32_t)c_loc : 4u * r4;
                         pd = keep_or_zero(pe, bits, pos);
-                        d = keep_or_zero(d, bits, pos) * a.rng.inv_keep;
+                        d = keep_or_zero(d, bits, pos);
                     }
                     pv[e] = pd;
                     dv[e] = pe * (d - del4[e]);
@@ -623,7 +626,9 @@ __global__ __launch_bounds__(kBwdThreads, (bwd_two_per_cu(DPAD, kDrop, KB) ? 2 :
             reinterpret_cast<T*>(a.dk) + b * a.dks[0] + (int64_t)kw0 * a.dks[1] + h * a.dks[2];
         T* dv_row0 =
             reinterpret_cast<T*>(a.dv) + b * a.dvs[0] + (int64_t)kw0 * a.dvs[1] + h * a.dvs[2];
-        store_block_via_lds<T, DPAD, kPitch>(dk_acc[0], a.scale, q_lds + wave * 32 * kPitch,
+        store_block_via_lds<T, DPAD, kPitch>(dk_acc[0],
+                                             kDrop != 0 ? a.scale * a.rng.inv_keep : a.scale,
+                                             q_lds + wave * 32 * kPitch,
                                              dk_row0, a.dks[1], a.sk - kw0, a.d);
         // with dropout: the factor 1 / (1 - p) that half_ds left out of P
         store_block_via_lds<T, DPAD, kPitch>(dv_acc[0], kDrop != 0 ? a.rng.inv_keep : 1.0f,

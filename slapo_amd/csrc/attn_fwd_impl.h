@@ -343,9 +343,10 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
             uint32_t mine = drop_bits;
             if constexpr (kDrop != 3) mine = draw_half(t * kBN + 32 * kb);
             const uint32_t mine_g = mine >> (kAccGroupStep * g);
+            // dropped probabilities become +0 (two instructions each); the factor 1 / (1 - p) of
+            // the kept ones goes onto the output rows when they are written
 #pragma unroll
-            for (int r = 0; r < 16; ++r)
-                s[r] = ((mine_g >> acc_row(r, 0)) & 1u) ? s[r] * a.rng.inv_keep : 0.f;
+            for (int r = 0; r < 16; ++r) s[r] = keep_or_zero(s[r], mine_g, acc_row(r, 0));
             drop_bits = mine;
 #pragma unroll
             for (int r2 = 0; r2 < 8; ++r2) pw[r2] = pack2<T>(s[2 * r2], s[2 * r2 + 1]);
@@ -494,7 +495,7 @@ __global__ __launch_bounds__(kThreads, (DPAD <= 64 && kDrop == 0 ? 3 : 2)) void 
 
     // ---- epilogue ----
     const float l_tot = sum_xor32(l_run);
-    const float inv_l = 1.0f / l_tot;
+    const float inv_l = kDrop != 0 ? a.rng.inv_keep / l_tot : 1.0f / l_tot;
     // every wavefront is past the last barrier of the loop: the K buffers are free, and each
     // wavefront routes its 32 output rows through its own quarter of them
     if (wq0 < a.sq) {
