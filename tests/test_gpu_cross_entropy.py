@@ -112,3 +112,37 @@ def test_shard_statistics_through_the_c_abi():
                                       rows, 10, 0, _lib.SLAPO_F32, st) == -4
     assert lib.slapo_amd_vocab_ce_bwd(P(shard), P(tgt), P(big_d), P(inv_d), P(go_d), P(grad), rows,
                                       10, 0, 1.0, _lib.SLAPO_F32, st) == -4
+
+
+@pytest.mark.parametrize("off_x,off_g", [(0, 0), (3, 3), (5, 1), (63, 63), (64, 8)])
+def test_rows_that_start_anywhere_relative_to_a_cache_line(off_x, off_g):
+    """The kernels align each row's vector body to a cache line and take the elements before
+    it one per thread; logits and gradient buffers whose bases differ modulo 16 bytes fall back
+    to element-wise accesses.  Buffers offset by a few elements, odd row length."""
+    lib = _lib.load()
+    g = torch.Generator().manual_seed(11)
+    rows, vocab = 19, 1237
+    logits = (torch.randn(rows, vocab, generator=g) * 3).to(torch.float16)
+    target = torch.randint(0, vocab, (rows,), generator=g)
+    go = torch.randn(rows, generator=g)
+    buf_x = torch.zeros(rows * vocab + 128, dtype=torch.float16, device="cuda")
+    buf_g = torch.full((rows * vocab + 128,), 7.0, dtype=torch.float16, device="cuda")
+    x = buf_x[off_x:off_x + rows * vocab].view(rows, vocab)
+    x.copy_(logits)
+    grad = buf_g[off_g:off_g + rows * vocab].view(rows, vocab)
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    out = torch.empty(4, rows, device="cuda")
+    tgt = target.cuda()
+    assert lib.slapo_amd_vocab_ce_fwd(P(x), P(tgt), P(out[0]), P(out[1]), P(out[2]), P(out[3]),
+                                      rows, vocab, 0, _lib.SLAPO_F16, st) == 0
+    ref = OC.shard_stats(logits.float(), target, 0)
+    for got, want in zip(out.cpu(), ref):
+        assert max_abs_err(got, want) <= 1e-4 * max(1.0, float(want.abs().max()))
+    inv = (1.0 / out[1]).contiguous()
+    assert lib.slapo_amd_vocab_ce_bwd(P(x), P(tgt), P(out[0]), P(inv), P(go.cuda()), P(grad), rows,
+                                      vocab, 0, 0.0, _lib.SLAPO_F16, st) == 0
+    _, softmax = OC.forward(logits, target)
+    assert_parity(grad, OC.backward(softmax, target, go.double()), torch.float16, "grad")
+    # nothing outside the gradient's own elements was written
+    assert bool((buf_g[:off_g] == 7.0).all()) and bool((buf_g[off_g + rows * vocab:] == 7.0).all())
