@@ -20,7 +20,10 @@ using namespace slapo;
 
 namespace {
 
-constexpr int kCeThreads = 256;
+// Threads per block (= per row).  Long rows take larger blocks: at 8192 x 50257 fp16 the forward
+// measured 130 / 123.5 / 147 us with 256 / 512 / 1024 threads (its block reduction grows with the
+// block) and the backward, which only streams, 307 / 293 / 279 us.
+constexpr int kCeMaxThreads = 1024;
 constexpr int kCeAlign = 128;  // bytes: alignment of a row's vector body
 
 // (m, s) pairs combine as  m = max(m1, m2),  s = s1 exp(m1 - m) + s2 exp(m2 - m); an empty
@@ -51,7 +54,7 @@ __device__ __forceinline__ RowSplit<T> split_row(const T* row, int n) {
         // 16-byte alignment only, the backward ran at 4.6 TB/s instead of 5.4 and the forward at
         // 6.2 instead of 6.5 at 8192 x 50257 fp16).  The head is at most 63 elements.
         constexpr int kPer = kCeAlign / (int)sizeof(T);
-        static_assert(kPer <= kCeThreads, "one thread per head element");
+        static_assert(kPer <= 256, "one thread per head element (smallest block)");
         const int mis = (int)((reinterpret_cast<uintptr_t>(row) & (kCeAlign - 1)) / sizeof(T));
         r.head = min(n, mis ? kPer - mis : 0);
         r.nvec = (n - r.head) / V;
@@ -67,7 +70,7 @@ struct CeVec {
 
 // Forward: m[row], s[row], predicted[row], sum_x[row] of one shard.  target may be any integer;
 // it counts when vocab_start <= target < vocab_start + n.
-template <typename T, int V>
+template <typename T, int V, int kCeThreads>
 __global__ __launch_bounds__(kCeThreads) void ce_fwd_kernel(
     const T* __restrict__ logits, const int64_t* __restrict__ target, float* __restrict__ m_out,
     float* __restrict__ s_out, float* __restrict__ pred_out, float* __restrict__ sumx_out, int n,
@@ -124,7 +127,7 @@ __global__ __launch_bounds__(kCeThreads) void ce_fwd_kernel(
         for (int u = 0; u < 4; ++u) take_vec(c[u]);
     }
     for (; i < sp.nvec; i += kCeThreads) take_vec(load_vec(i));
-    // block reduction: butterflies inside the wavefront, then the four wavefronts through LDS
+    // block reduction: butterflies inside the wavefront, then the block's wavefronts through LDS
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) {
         const float m2 = __shfl_xor(m, off, 64);
@@ -157,7 +160,7 @@ __global__ __launch_bounds__(kCeThreads) void ce_fwd_kernel(
 // Backward: grad[row, v] = g[row] (exp(x - M[row]) inv_s[row] - onehot_scale [v == target] - flat)
 // with M, inv_s the combined maximum and 1 / sum of the whole vocabulary, onehot_scale =
 // 1 - smoothing and flat = smoothing / n (slapo/op/cross_entropy.py:100-122).
-template <typename T, int V>
+template <typename T, int V, int kCeThreads>
 __global__ __launch_bounds__(kCeThreads) void ce_bwd_kernel(
     const T* __restrict__ logits, const int64_t* __restrict__ target,
     const float* __restrict__ row_max, const float* __restrict__ inv_sum,
@@ -229,9 +232,15 @@ inline bool ce_dims_ok(int64_t rows, int64_t n) {
 template <typename T>
 int ce_fwd_dispatch(const void* logits, const int64_t* target, float* m, float* s, float* pred,
                     float* sumx, int64_t rows, int64_t n, int64_t vocab_start, hipStream_t st) {
-    hipLaunchKernelGGL((ce_fwd_kernel<T, Elem<T>::kPerVec>), dim3((unsigned)rows),
-                       dim3(kCeThreads), 0, st, (const T*)logits, target, m, s, pred, sumx,
-                       (int)n, vocab_start);
+#define SLAPO_CE_FWD(THREADS)                                                                   \
+    hipLaunchKernelGGL((ce_fwd_kernel<T, Elem<T>::kPerVec, THREADS>), dim3((unsigned)rows),     \
+                       dim3(THREADS), 0, st, (const T*)logits, target, m, s, pred, sumx, (int)n, \
+                       vocab_start)
+    if (n >= 16384)
+        SLAPO_CE_FWD(512);
+    else
+        SLAPO_CE_FWD(256);
+#undef SLAPO_CE_FWD
     return check_launch();
 }
 
@@ -244,14 +253,19 @@ int ce_bwd_dispatch(const void* logits, const int64_t* target, const float* row_
     // otherwise every element goes through the scalar path.
     const bool same = ((reinterpret_cast<uintptr_t>(logits) ^ reinterpret_cast<uintptr_t>(grad)) &
                        15) == 0;
-    if (same)
-        hipLaunchKernelGGL((ce_bwd_kernel<T, Elem<T>::kPerVec>), dim3((unsigned)rows),
-                           dim3(kCeThreads), 0, st, (const T*)logits, target, row_max, inv_sum,
-                           grad_loss, (T*)grad, (int)n, vocab_start, onehot_scale, flat);
+#define SLAPO_CE_BWD(VEC, THREADS)                                                              \
+    hipLaunchKernelGGL((ce_bwd_kernel<T, VEC, THREADS>), dim3((unsigned)rows), dim3(THREADS), 0, \
+                       st, (const T*)logits, target, row_max, inv_sum, grad_loss, (T*)grad,      \
+                       (int)n, vocab_start, onehot_scale, flat)
+    if (!same)
+        SLAPO_CE_BWD(1, 256);
+    else if (n >= 32768)
+        SLAPO_CE_BWD(Elem<T>::kPerVec, kCeMaxThreads);
+    else if (n >= 8192)
+        SLAPO_CE_BWD(Elem<T>::kPerVec, 512);
     else
-        hipLaunchKernelGGL((ce_bwd_kernel<T, 1>), dim3((unsigned)rows), dim3(kCeThreads), 0, st,
-                           (const T*)logits, target, row_max, inv_sum, grad_loss, (T*)grad,
-                           (int)n, vocab_start, onehot_scale, flat);
+        SLAPO_CE_BWD(Elem<T>::kPerVec, 256);
+#undef SLAPO_CE_BWD
     return check_launch();
 }
 

@@ -27,11 +27,13 @@ def _case(shape, vocab, dtype, seed=2013, scale=3.0):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("shape,vocab", [((4, 6), 50257), ((33,), 1000), ((2, 3), 8), ((5,), 1),
-                                         ((3, 2), 4099), ((2,), 70000)])
+                                         ((3, 2), 4099), ((2,), 70000), ((3,), 12289),
+                                         ((2, 2), 20001)])
 @pytest.mark.parametrize("alpha", [0.0, 0.1])
 def test_loss_and_gradient(dtype, shape, vocab, alpha):
     """Unpadded vocabularies (rows start at every element offset: head / body / tail paths),
-    tiny and single-class rows, label smoothing."""
+    tiny and single-class rows, label smoothing; row lengths on both sides of the thresholds at
+    which the kernels take larger blocks (8192, 16384, 32768)."""
     if alpha > 0 and vocab < 2:
         pytest.skip("label smoothing needs two classes")
     logits, target, go = _case(shape, vocab, dtype)
