@@ -70,7 +70,7 @@ typedef struct slapo_dropout_plan {
     int32_t vec;              /* elements handled per subsequence per loop trip: 1,2,4,8,16     */
     int32_t calls_per_iter;   /* Philox calls per loop trip = ceil(vec/4) (1 when vec == 1)     */
     int64_t offset_increment; /* amount the generator's offset must be advanced after the draw */
-    const void* rng_state;    /* NULL, or a device address of two uint64 {seed, offset}: see below */
+    const void* rng_state;    /* NULL, or a device address of two uint64 {seed, offset}: see above */
 } slapo_dropout_plan;
 
 /* Host Philox4x32-10 block function (10 rounds).  Pure host code; usable without a GPU. */
