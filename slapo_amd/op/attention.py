@@ -28,7 +28,8 @@ import torch
 import torch.nn.functional as F
 from torch import nn
 
-from ..random import draw_philox, draw_philox_state
+from ..random import draw_philox  # noqa: F401  (kept importable from here for direct launches)
+from ..random import draw_philox_state
 from . import _kernels as K
 from .fused_bias import bias_dropout
 
