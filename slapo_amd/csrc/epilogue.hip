@@ -235,10 +235,17 @@ __device__ __forceinline__ void colsum_walk(int64_t rows, int64_t cols, float* _
     for (int i = 0; i < V; ++i) acc[i] = 0.f;
     const int64_t r_begin = (int64_t)blockIdx.y * rows_per_block;
     if (active) {
+        if (r_begin + rows_per_block <= rows) {
+            // a whole block of rows: no test between the iterations, so that the loads of an
+            // unrolled group of four rows are requested together
 #pragma unroll 4
-        for (int it = 0; it < rows_per_block / kRowLanes; ++it) {
-            const int64_t r = r_begin + ry + (int64_t)it * kRowLanes;
-            if (r < rows) body(r, col0, acc);
+            for (int it = 0; it < rows_per_block / kRowLanes; ++it)
+                body(r_begin + ry + (int64_t)it * kRowLanes, col0, acc);
+        } else {
+            for (int it = 0; it < rows_per_block / kRowLanes; ++it) {
+                const int64_t r = r_begin + ry + (int64_t)it * kRowLanes;
+                if (r < rows) body(r, col0, acc);
+            }
         }
     }
     if (!want_sum) return;
