@@ -328,6 +328,7 @@ __global__ __launch_bounds__(256) void bias_dropout_bwd_kernel(const T* __restri
 // through LDS.  Many small blocks: the stage is latency bound, not bandwidth bound.
 constexpr int kFinCols = 16;
 constexpr int kFinRows = 16;
+constexpr int kFinWide = 32;  // loads in flight per thread in the wide stage of a finishing kernel
 template <typename T>
 __global__ __launch_bounds__(256) void colsum_finish_kernel(const float* __restrict__ partial,
                                                             T* __restrict__ dbias,
@@ -340,6 +341,17 @@ __global__ __launch_bounds__(256) void colsum_finish_kernel(const float* __restr
     if (c < cols) {
         float t0 = 0.f, t1 = 0.f, t2 = 0.f, t3 = 0.f;
         int64_t k = ry;
+        // many partial rows (narrow matrices in blocks of 16 rows): 32 loads in flight per thread,
+        // the stage is a chain of memory round trips (bias-dropout backward at bf16 8192 x 1024:
+        // 14.5 -> 13.2 us with its finishing kernel)
+        for (; k + (kFinWide - 1) * kFinRows < n_partials; k += kFinWide * kFinRows) {
+            float v[kFinWide];
+#pragma unroll
+            for (int j = 0; j < kFinWide; ++j) v[j] = partial[(k + j * kFinRows) * cols + c];
+#pragma unroll
+            for (int j = 0; j < kFinWide; j += 4)
+                t0 += v[j], t1 += v[j + 1], t2 += v[j + 2], t3 += v[j + 3];
+        }
         for (; k + 3 * kFinRows < n_partials; k += 4 * kFinRows) {
             t0 += partial[k * cols + c];
             t1 += partial[(k + kFinRows) * cols + c];
@@ -711,9 +723,16 @@ __global__ __launch_bounds__(256) void ln_finish_kernel(const float* __restrict_
     const int64_t c = (int64_t)blockIdx.x * kFC + cx;
     float t = 0.f;
     if (c < cols3) {
-        // eight loads in flight per thread
+        // 32 loads in flight per thread while that many rows are left, then eight
         float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
         int64_t k = ry;
+        for (; k + (kFinWide - 1) * kFR < n_partials; k += kFinWide * kFR) {
+            float v[kFinWide];
+#pragma unroll
+            for (int j = 0; j < kFinWide; ++j) v[j] = partial[(k + j * kFR) * cols3 + c];
+#pragma unroll
+            for (int j = 0; j < kFinWide; ++j) acc[j & 7] += v[j];
+        }
         for (; k + 7 * kFR < n_partials; k += 8 * kFR) {
             float v[8];
 #pragma unroll
