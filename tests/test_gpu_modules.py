@@ -151,3 +151,54 @@ def test_replaced_children_of_the_tail_are_called_as_modules():
 
     m.out_proj = Wrapped(m.out_proj)
     assert torch.equal(m(x)[0], no_drop + 1)
+
+
+def test_ops_on_side_streams_from_two_threads():
+    """The entry points take the caller's stream and keep no state between calls: two host
+    threads, each on a stream of its own (default priority), run attention forward + backward and
+    the LayerNorm epilogue at the same time and get what a single-threaded run on the default
+    stream gets, bit for bit."""
+    import threading
+
+    from slapo_amd import op
+
+    g = torch.Generator().manual_seed(21)
+    mk = lambda *s: torch.randn(*s, generator=g).to(torch.bfloat16).cuda()
+    cases = []
+    for d in (64, 128):
+        q, k, v, do = (mk(2, 384, 4, d) for _ in range(4))
+        x, res, gy, w, b = mk(384, 512), mk(384, 512), mk(384, 512), mk(512), mk(512)
+        cases.append((q, k, v, do, x, res, gy, w, b))
+
+    def run(case):
+        q, k, v, do, x, res, gy, w, b = case
+        ql, kl, vl, xl = (t.clone().requires_grad_(True) for t in (q, k, v, x))
+        out = op.hip_attention(ql, kl, vl, None, causal=True)
+        y = op.bias_dropout_residual_layer_norm(xl, b, res, w, b, 0.0, 1e-5, True)
+        grads = torch.autograd.grad((out, y), (ql, kl, vl, xl), (do, gy))
+        return (out, y) + tuple(grads)
+
+    want = [run(c) for c in cases]
+    torch.cuda.synchronize()
+    got, errors = [None, None], []
+
+    def worker(i):
+        try:
+            stream = torch.cuda.Stream()
+            with torch.cuda.stream(stream):
+                for _ in range(5):
+                    res_ = run(cases[i])
+                stream.synchronize()
+            got[i] = res_
+        except Exception as exc:  # pylint: disable=broad-except
+            errors.append(exc)
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(60)
+    assert not errors, errors
+    for i in range(2):
+        for a, b_ in zip(got[i], want[i]):
+            assert torch.equal(a, b_)
