@@ -646,3 +646,25 @@ def test_random_configurations_against_the_oracle(seed):
     print(f"seed {seed}: {dtype} b{b} h{h} sq{sq} sk{sk} d{d} causal={causal} window={window} "
           f"mask={layout} p={p}", flush=True)
     _check(q, k, v, do, mask, causal, window, dtype, p=p)
+
+
+@pytest.mark.parametrize("shape,causal,window", [((1, 16384, 1, 64), True, 0),
+                                                 ((1, 8192, 2, 128), True, 0),
+                                                 ((1, 8192, 1, 80), False, 0),
+                                                 ((1, 12288, 1, 128), True, 1000)])
+def test_long_sequences_against_the_fp32_kernels(shape, causal, window):
+    """Sequence lengths well beyond the benchmark's (16 to 256 key tiles per workgroup, offsets
+    past 2^24 elements within a head): the MFMA kernels against the fp32 FMA kernels of this
+    library (oracle-checked at 1e-5 on small shapes) on the same bf16 values, at the 2e-2 bar."""
+    g = torch.Generator().manual_seed(77)
+    mk = lambda: torch.randn(*shape, generator=g).to(torch.bfloat16)
+    q, k, v, do = mk(), mk(), mk(), mk()
+    outs = {}
+    for kind, cast in (("mfma", torch.bfloat16), ("fma", torch.float32)):
+        qd, kd, vd = (t.to(cast).cuda().requires_grad_(True) for t in (q, k, v))
+        out = op.hip_attention(qd, kd, vd, None, causal=causal, window=window)
+        out.backward(do.to(cast).cuda())
+        outs[kind] = (out.detach(), qd.grad, kd.grad, vd.grad)
+    for name, a, r in zip(("out", "dq", "dk", "dv"), outs["mfma"], outs["fma"]):
+        err, top = max_abs_err(a, r), r.abs().max().item()
+        assert err <= 2e-2 * top + 1e-5, f"{name}: {err:.3e} > 2e-2 x {top:.3e}"
